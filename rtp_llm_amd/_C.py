@@ -15,11 +15,11 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355_decode_tuning.so" if TUNING else
 OK, ERR_ARG, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = 0, -1, -2, -3, -4
 W4, W8, W16 = 4, 8, 16
 KV_FP16, KV_INT8, KV_BF16 = 0, 1, 2
-ACT_F16, ACT_BF16 = 0, 1
+ACT_F16, ACT_BF16, ACT_F32 = 0, 1, 2
 EPI_NONE, EPI_SILU_MUL, EPI_OUT_F32, EPI_OUT_IMAGE = 0, 1, 2, 4
 PF_QKV, PF_O, PF_GATE_UP, PF_QKV_LATE, PF_O_LATE, PF_TP_COMM, PF_TP_INLAUNCH, PF_QKV_IN_FOLD = 1, 2, 4, 16, 32, 64, 128, 256   # mi355_decoder_set_weight_prefetch mask bits
 HINT_STAGED, HINT_NO_PERSISTENT = 0x100, 0x200
-ABI_VERSION = 3
+ABI_VERSION = 4
 KC_NAMES = ["gemm_quant", "gemm_lmhead", "attn", "rope_kv", "norm", "other", "comm"]
 
 vp, i32, f32, sz = C.c_void_p, C.c_int32, C.c_float, C.c_size_t
@@ -158,7 +158,24 @@ SIGNATURES = {
     "mi355_decoder_oob_count": (C.c_int64, [vp, vp]),
 }
 
+# libmi355_hybrid.so: dense linears on [out, in] weights + the kernels of the hybrid decoder family (a library of its own, so that a
+# process serving such a model builds and loads nothing else)
+HYBRID_LIB_PATH = os.path.join(_HERE, "lib", "libmi355_hybrid.so")
+ip = C.POINTER(i32)
+HYBRID_SIGNATURES = {
+    "mi355_abi_version": (i32, []),
+    "mi355_last_error": (C.c_char_p, []),
+    "mi355_dense_linear": (i32, [vp, i32, i32, vp, i32, i32, vp, vp, i32, i32, i32, i32, f32, i32, vp]),
+    "mi355_hy_embed": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
+    "mi355_hy_residual_norm": (i32, [vp, vp, vp, f32, vp, i32, i32, vp, vp, f32, f32, vp, vp, i32, vp]),
+    "mi355_hy_attn_prep": (i32, [vp, i32, i32, i32, ip, vp, vp, i32, f32, vp, vp, vp, i32, vp, vp, i32, vp]),
+    "mi355_hy_attn_rows": (i32, [vp, i32, f32, ip, i32, i32, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp]),
+    "mi355_hy_scan": (i32, [i32, vp, i32, i32, i32, i32, vp, i32, vp, vp, f32, f32, i32, i32, i32, vp, vp, vp, i32, vp, vp, i32, vp]),
+    "mi355_hy_head_norm": (i32, [vp, i32, i32, i32, vp, f32, vp, i32, i32, vp, i32, vp]),
+}
+
 _lib = None
+_hybrid = None
 
 
 class Mi355Error(RuntimeError):
@@ -183,6 +200,30 @@ def lib():
             raise Mi355Error("libmi355_decode.so ABI version mismatch")
         _lib = l
     return _lib
+
+
+def hybrid_lib():
+    """Load libmi355_hybrid.so (once).  Raises if it has not been built: no fallback."""
+    global _hybrid
+    if _hybrid is None:
+        if not os.path.exists(HYBRID_LIB_PATH):
+            raise Mi355Error(f"{HYBRID_LIB_PATH} not found - build it with `python -m rtp_llm_amd.build --hybrid` "
+                             "(the HIP extension is required; there is no CPU fallback)")
+        import torch  # noqa: F401  (the HIP runtime PyTorch bundles must be the one this library binds to)
+        l = C.CDLL(HYBRID_LIB_PATH)
+        for name, (res, args) in HYBRID_SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype, fn.argtypes = res, args
+        if l.mi355_abi_version() != ABI_VERSION:
+            raise Mi355Error("libmi355_hybrid.so ABI version mismatch")
+        _hybrid = l
+    return _hybrid
+
+
+def check_hybrid(rc: int, what: str = "") -> int:
+    if rc < 0:
+        raise Mi355Error(f"{what}: mi355 error {rc}: {hybrid_lib().mi355_last_error().decode(errors='replace')}")
+    return rc
 
 
 def check(rc: int, what: str = "") -> int:

@@ -1,0 +1,333 @@
+// Dense linear layers on weights kept in checkpoint layout: y[M, N] = x[M, K] . W[N, K]^T with W row-major [out, in].
+//
+// Both operands are contiguous along K, which is the layout v_mfma_f32_16x16x32_bf16 wants for its A and B fragments (8 consecutive k per
+// lane), so no weight image is built: a model whose layers have many small, differently shaped projections (recurrent gates, low-rank
+// decays, shared-KV attention) loads its tensors as they are.  Three kernels, all with fp32 accumulation and an fp32 epilogue:
+//   * tile kernel, bf16:  64 x 128 block tile, 4 waves of 32 x 64, K staged through LDS 64 at a time, MFMA 16x16x32;
+//   * tile kernel, fp32:  64 x 64 block tile, 4 x 4 register micro-tiles, true fp32 FMAs (no reduced-precision matrix mode);
+//   * row kernel (M <= 16): one wave per output column streams its weight row once, 16-byte loads, wave reduction at the end.
+// Epilogues: bias, gated activation act(gate) * up (weight rows grouped [32 gate | 32 up], so one lane holds both), tanh soft cap.
+// Output is fp32 or the activation type.  A result row depends only on its own input row: the k order of the accumulation is fixed by
+// the kernel, never by M or by the row's place in the batch.
+#include "common.h"
+
+namespace {
+
+constexpr int DN_ACT_NONE = 0, DN_ACT_RELU = 1, DN_ACT_SILU = 2;
+
+struct DenseParams {
+    const void* x; const void* w; const void* bias; void* y;
+    int M, N, K, ldx, ldy;
+    int gated;       // 0: N outputs; 1: rows of w are [32 gate | 32 up] groups, N / 2 outputs
+    int act;         // DN_ACT_* applied to the gate
+    int out_f32;
+    float softcap;   // > 0: y = cap * tanh(y / cap)
+    int vec;         // 16-byte loads allowed (alignment and K % 8 == 0 checked on the host)
+};
+
+__device__ __forceinline__ float dn_act(float g, int act) {
+    if (act == DN_ACT_RELU) return g > 0.f ? g : 0.f;
+    if (act == DN_ACT_SILU) return g / (1.f + __expf(-g));
+    return g;
+}
+
+template <typename T> __device__ __forceinline__ float dn_ld(const T* p) { return (float)*p; }
+
+template <typename T>
+__device__ __forceinline__ void dn_store(const DenseParams& p, int row, int col, float v) {
+    if (p.softcap > 0.f) v = p.softcap * tanhf(v / p.softcap);
+    if (p.out_f32) ((float*)p.y)[(size_t)row * p.ldy + col] = v;
+    else           ((T*)p.y)[(size_t)row * p.ldy + col] = (T)v;
+}
+
+// ------------------------------------------------------------------------------------------------ bf16 tile kernel
+constexpr int TB_M = 64, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;   // LDS row stride in elements (144 bytes: 16-byte aligned)
+
+__device__ __forceinline__ u32x4 dn_chunk_bf16(const bf16* base, int row, int rows, int k, int K, int ld, int vec) {
+    u32x4 z = {0u, 0u, 0u, 0u};
+    if (row >= rows || k >= K) return z;
+    const bf16* p = base + (size_t)row * ld + k;
+    if (vec) return *(const u32x4*)p;
+    uint16_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) e[i] = (k + i < K) ? __builtin_bit_cast(uint16_t, p[i]) : (uint16_t)0;
+    u32x4 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (uint32_t)e[2 * i] | ((uint32_t)e[2 * i + 1] << 16);
+    return r;
+}
+
+__global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
+    __shared__ __attribute__((aligned(16))) bf16 As[TB_M * TB_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Bs[TB_N * TB_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;                       // wave tile: rows wm*32.., cols wn*64..
+    const int m0 = blockIdx.y * TB_M, n0 = blockIdx.x * TB_N;
+    const bf16* X = (const bf16*)p.x;
+    const bf16* W = (const bf16*)p.w;
+    f32x4 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // staging: chunk c of 8 elements; A has 64 x 8 chunks (2 per thread), B 128 x 8 (4 per thread)
+    u32x4 ra[2], rb[4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { const int c = tid + i * 256; ra[i] = dn_chunk_bf16(X, m0 + (c >> 3), p.M, k0 + (c & 7) * 8, p.K, p.ldx, p.vec); }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { const int c = tid + i * 256; rb[i] = dn_chunk_bf16(W, n0 + (c >> 3), p.N, k0 + (c & 7) * 8, p.K, p.K, p.vec); }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < p.K; k0 += TB_K) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) { const int c = tid + i * 256; *(u32x4*)&As[(c >> 3) * TB_LD + (c & 7) * 8] = ra[i]; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { const int c = tid + i * 256; *(u32x4*)&Bs[(c >> 3) * TB_LD + (c & 7) * 8] = rb[i]; }
+        __syncthreads();
+        if (k0 + TB_K < p.K) fetch(k0 + TB_K);
+#pragma unroll
+        for (int ks = 0; ks < TB_K; ks += 32) {
+            const int kk = ks + (lane >> 4) * 8, r = lane & 15;
+            bf16x8 a[2], b[4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = *(const bf16x8*)&As[(wm * 32 + i * 16 + r) * TB_LD + kk];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)&Bs[(wn * 64 + j * 16 + r) * TB_LD + kk];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // C fragment: lane holds column (lane & 15), rows 4 * (lane >> 4) + e
+    const int cl = lane & 15, rq = (lane >> 4) * 4;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = m0 + wm * 32 + i * 16 + rq + e;
+            if (row >= p.M) continue;
+            if (p.gated) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int ng = n0 + wn * 64 + j * 16 + cl;         // weight row of the gate; its up row is ng + 32
+                    if (ng + 32 >= p.N) continue;
+                    float g = acc[i][j][e], u = acc[i][j + 2][e];
+                    if (p.bias) { g += dn_ld((const bf16*)p.bias + ng); u += dn_ld((const bf16*)p.bias + ng + 32); }
+                    dn_store<bf16>(p, row, (ng >> 6) * 32 + (ng & 31), dn_act(g, p.act) * u);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = n0 + wn * 64 + j * 16 + cl;
+                    if (n >= p.N) continue;
+                    float v = acc[i][j][e];
+                    if (p.bias) v += dn_ld((const bf16*)p.bias + n);
+                    dn_store<bf16>(p, row, n, dn_act(v, p.act));
+                }
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------------ fp32 tile kernel
+constexpr int TF_M = 64, TF_N = 64, TF_K = 16, TF_LD = 68;
+
+__device__ __forceinline__ f32x4 dn_chunk_f32(const float* base, int row, int rows, int k, int K, int ld, int vec) {
+    f32x4 r = {0.f, 0.f, 0.f, 0.f};
+    if (row >= rows || k >= K) return r;
+    const float* p = base + (size_t)row * ld + k;
+    if (vec) return *(const f32x4*)p;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = (k + i < K) ? p[i] : 0.f;
+    return r;
+}
+
+__global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
+    __shared__ __attribute__((aligned(16))) float As[TF_K * TF_LD];   // [k][m]
+    __shared__ __attribute__((aligned(16))) float Bs[TF_K * TF_LD];   // [k][n]
+    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+    const int m0 = blockIdx.y * TF_M, n0 = blockIdx.x * TF_N;
+    const float* X = (const float*)p.x;
+    const float* W = (const float*)p.w;
+    float acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    const int lr = tid >> 2, lk = (tid & 3) * 4;          // staging: row lr, k offset lk
+    f32x4 ra = dn_chunk_f32(X, m0 + lr, p.M, lk, p.K, p.ldx, p.vec);
+    f32x4 rb = dn_chunk_f32(W, n0 + lr, p.N, lk, p.K, p.K, p.vec);
+    for (int k0 = 0; k0 < p.K; k0 += TF_K) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { As[(lk + i) * TF_LD + lr] = ra[i]; Bs[(lk + i) * TF_LD + lr] = rb[i]; }
+        __syncthreads();
+        if (k0 + TF_K < p.K) {
+            ra = dn_chunk_f32(X, m0 + lr, p.M, k0 + TF_K + lk, p.K, p.ldx, p.vec);
+            rb = dn_chunk_f32(W, n0 + lr, p.N, k0 + TF_K + lk, p.K, p.K, p.vec);
+        }
+#pragma unroll
+        for (int k = 0; k < TF_K; ++k) {
+            const f32x4 a = *(const f32x4*)&As[k * TF_LD + ty * 4];
+            const float b0 = Bs[k * TF_LD + 2 * tx], b1 = Bs[k * TF_LD + 2 * tx + 1];
+            const float b2 = Bs[k * TF_LD + 32 + 2 * tx], b3 = Bs[k * TF_LD + 32 + 2 * tx + 1];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i][0] = __builtin_fmaf(a[i], b0, acc[i][0]); acc[i][1] = __builtin_fmaf(a[i], b1, acc[i][1]);
+                acc[i][2] = __builtin_fmaf(a[i], b2, acc[i][2]); acc[i][3] = __builtin_fmaf(a[i], b3, acc[i][3]);
+            }
+        }
+    }
+    // thread columns: {2 tx, 2 tx + 1} of the first 32 and the same of the second 32 (gate / up of one channel under `gated`)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = m0 + ty * 4 + i;
+        if (row >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + 2 * tx + j;
+            if (p.gated) {
+                if (n + 32 >= p.N) continue;
+                float g = acc[i][j], u = acc[i][j + 2];
+                if (p.bias) { g += ((const float*)p.bias)[n]; u += ((const float*)p.bias)[n + 32]; }
+                dn_store<float>(p, row, (n >> 6) * 32 + (n & 31), dn_act(g, p.act) * u);
+            } else {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int nn = n + 32 * h;
+                    if (nn >= p.N) continue;
+                    float v = acc[i][j + 2 * h];
+                    if (p.bias) v += ((const float*)p.bias)[nn];
+                    dn_store<float>(p, row, nn, dn_act(v, p.act));
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ row kernel (small M)
+template <typename T> struct DnVec;
+template <> struct DnVec<bf16> {
+    static constexpr int W = 8;
+    static __device__ __forceinline__ void load(const bf16* p, int n, int vec, float (&o)[8]) {
+        if (vec && n >= 8) { act_unpack8<true>(*(const u32x4*)p, o); return; }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = i < n ? (float)p[i] : 0.f;
+    }
+};
+template <> struct DnVec<float> {
+    static constexpr int W = 8;
+    static __device__ __forceinline__ void load(const float* p, int n, int vec, float (&o)[8]) {
+        if (vec && n >= 8) {
+            const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = i < n ? p[i] : 0.f;
+    }
+};
+
+__device__ __forceinline__ float dn_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// One wave per output: a plain column n, or under `gated` one channel c (gate row and up row).  MR rows of x per pass.
+template <typename T, int MR>
+__global__ __launch_bounds__(256) void dense_rows_kernel(DenseParams p, int mbase) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int o = blockIdx.x * 4 + wave;
+    const int nout = p.gated ? p.N / 2 : p.N;
+    if (o >= nout) return;
+    const int n0 = p.gated ? (o >> 5) * 64 + (o & 31) : o;
+    const T* X = (const T*)p.x;
+    const T* W0 = (const T*)p.w + (size_t)n0 * p.K;
+    const T* W1 = W0 + (size_t)32 * p.K;
+    const int rows = min(MR, p.M - mbase);
+    float a0[MR], a1[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) { a0[m] = 0.f; a1[m] = 0.f; }
+    for (int k = lane * 8; k < p.K; k += 64 * 8) {
+        float w0[8], w1[8], xv[8];
+        DnVec<T>::load(W0 + k, p.K - k, p.vec, w0);
+        if (p.gated) DnVec<T>::load(W1 + k, p.K - k, p.vec, w1);
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+            if (m >= rows) break;
+            DnVec<T>::load(X + (size_t)(mbase + m) * p.ldx + k, p.K - k, p.vec, xv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a0[m] = __builtin_fmaf(xv[i], w0[i], a0[m]);
+            if (p.gated) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a1[m] = __builtin_fmaf(xv[i], w1[i], a1[m]);
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        if (m >= rows) break;
+        float g = dn_wave_sum(a0[m]);
+        float u = p.gated ? dn_wave_sum(a1[m]) : 0.f;
+        if (lane != 0) continue;
+        if (p.bias) { g += dn_ld((const T*)p.bias + n0); if (p.gated) u += dn_ld((const T*)p.bias + n0 + 32); }
+        g = dn_act(g, p.act);
+        dn_store<T>(p, mbase + m, o, p.gated ? g * u : g);
+    }
+}
+
+} // namespace
+
+// x [M, K] (row stride ldx) and w [N, K] of act_dtype (MI355_ACT_BF16 or MI355_ACT_F32); bias [N] of act_dtype or null;
+// y [M, N or N / 2] fp32 (out_f32) or act_dtype, row stride ldy.  gated: the N weight rows are groups of 64 = 32 gate rows followed by
+// the 32 up rows of the same channels (N % 64 == 0); y[m, c] = act(gate_c) * up_c.  act: 0 none, 1 relu, 2 silu (on the gate, or on
+// the plain output).  softcap > 0: y <- softcap * tanh(y / softcap).
+extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias,
+                                  void* y, int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, float softcap,
+                                  int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && ldx >= K, "dense_linear: M=%d N=%d K=%d ldx=%d", M, N, K, ldx);
+    MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_linear: act_dtype=%d (bf16 or fp32)", act_dtype);
+    MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_linear: gated needs N %% 64 == 0 (N=%d)", N);
+    MI355_CHECK_ARG(act >= 0 && act <= 2, "dense_linear: act=%d", act);
+    MI355_CHECK_ARG(ldy >= (gated ? N / 2 : N), "dense_linear: ldy=%d", ldy);
+    const bool bf = act_dtype == MI355_ACT_BF16;
+    const size_t es = bf ? 2 : 4;
+    DenseParams p;
+    p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
+    p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
+    p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    (void)es;
+    hipStream_t st = (hipStream_t)stream;
+    if (M <= 16) {
+        const int nout = gated ? N / 2 : N;
+        const dim3 grid((nout + 3) / 4);
+        for (int mb = 0; mb < M; mb += 8) {
+            const int r = M - mb;
+            if (bf) {
+                if (r <= 2)      hipLaunchKernelGGL((dense_rows_kernel<bf16, 2>), grid, dim3(256), 0, st, p, mb);
+                else if (r <= 4) hipLaunchKernelGGL((dense_rows_kernel<bf16, 4>), grid, dim3(256), 0, st, p, mb);
+                else             hipLaunchKernelGGL((dense_rows_kernel<bf16, 8>), grid, dim3(256), 0, st, p, mb);
+            } else {
+                if (r <= 2)      hipLaunchKernelGGL((dense_rows_kernel<float, 2>), grid, dim3(256), 0, st, p, mb);
+                else if (r <= 4) hipLaunchKernelGGL((dense_rows_kernel<float, 4>), grid, dim3(256), 0, st, p, mb);
+                else             hipLaunchKernelGGL((dense_rows_kernel<float, 8>), grid, dim3(256), 0, st, p, mb);
+            }
+        }
+        MI355_CHECK_LAUNCH("dense_rows_kernel");
+        return MI355_OK;
+    }
+    if (bf) {
+        const dim3 grid((N + TB_N - 1) / TB_N, (M + TB_M - 1) / TB_M);
+        hipLaunchKernelGGL(dense_tile_bf16_kernel, grid, dim3(256), 0, st, p);
+        MI355_CHECK_LAUNCH("dense_tile_bf16_kernel");
+    } else {
+        const dim3 grid((N + TF_N - 1) / TF_N, (M + TF_M - 1) / TF_M);
+        hipLaunchKernelGGL(dense_tile_f32_kernel, grid, dim3(256), 0, st, p);
+        MI355_CHECK_LAUNCH("dense_tile_f32_kernel");
+    }
+    return MI355_OK;
+}

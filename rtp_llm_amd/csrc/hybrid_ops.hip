@@ -1,0 +1,439 @@
+// Kernels of the hybrid decoder family: layers x <- x + m * (mixer(norm1 x) + ffn(norm2 x)) over an fp32 residual stream, whose token mixer is
+// either paged attention (chunk-local causal mask, optional sink in the softmax denominator, unit-normed values that are rotated by their
+// position and turned back at the query's position) or a gated linear recurrence S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with
+// its state in fp32 slots (HGRN2 and gated-linear-attention parametrisations of a, k, q).
+//
+// One ragged batch of rows serves prefill portions and decode tokens alike: every row carries its position and the index of its
+// sequence; a sequence carries its block-table row, its state slot and the range of its rows.  What the model states as 32-bit is fp32
+// here whatever the activation type T (bf16 or float): positions and angles, scores and softmax, norms, gates, decays, states, residual.
+#include "common.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ void hy_load8(const T* p, float (&o)[8]);
+template <> __device__ __forceinline__ void hy_load8<bf16>(const bf16* p, float (&o)[8]) { act_unpack8<true>(*(const u32x4*)p, o); }
+template <> __device__ __forceinline__ void hy_load8<float>(const float* p, float (&o)[8]) {
+    const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
+}
+
+__device__ __forceinline__ float hy_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float hy_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float hy_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float hy_silu(float z) { return z / (1.f + expf(-z)); }
+
+// channel indices of rotation pair i under a layout: 0 = interleaved (2i, 2i+1), 1 = halves (i, i + n/2)
+__device__ __forceinline__ void hy_pair(int layout, int i, int n, int& c0, int& c1) {
+    if (layout == 0) { c0 = 2 * i; c1 = 2 * i + 1; } else { c0 = i; c1 = i + n / 2; }
+}
+
+// ------------------------------------------------------------------------------------------------ embedding -> fp32 stream
+template <typename T>
+__global__ __launch_bounds__(256) void hy_embed_kernel(const int32_t* ids, const T* table, int W, int vocab, float* out) {
+    const int r = blockIdx.x;
+    int id = ids[r];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int c = threadIdx.x; c < W; c += 256) out[(size_t)r * W + c] = (float)table[(size_t)id * W + c];
+}
+
+// ------------------------------------------------------------------------------------------------ residual update + one or two norms
+// x[src] <- x[src] + mult * (a[src] + b[src]) (written back unless rows are gathered), then h1 = norm(x) * (off + w1), h2 likewise.
+template <typename T>
+__global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, float mult, const int32_t* rows,
+                                                               const T* w1, const T* w2, float off, float eps, int W, T* h1, T* h2) {
+    extern __shared__ float hy_xs[];
+    __shared__ float red[4];
+    const int r = blockIdx.x, src = rows ? rows[r] : r;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const size_t i = (size_t)src * W + c;
+        float v = x[i];
+        if (a || b) {
+            const float y = (a ? a[i] : 0.f) + (b ? b[i] : 0.f);
+            v = v + mult * y;
+            if (!rows) x[i] = v;
+        }
+        hy_xs[c] = v;
+        ss = __builtin_fmaf(v, v, ss);
+    }
+    ss = hy_wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float u = hy_xs[c] * inv;
+        if (h1) h1[(size_t)r * W + c] = (T)(u * (off + (float)w1[c]));
+        if (h2) h2[(size_t)r * W + c] = (T)(u * (off + (float)w2[c]));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ attention: rotate q in place, write K / V pages
+struct AttnGeom {
+    int H, G, dim, vdim;
+    int rot_dims, rot_layout;     // rotary span of q / k heads (0 = none) and its pair layout
+    int v_layout;                 // pair layout of the value rotation
+    int page, max_blocks, num_pages;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, int koff, int voff, AttnGeom g, const float* kfreq, const float* vfreq,
+                                                           int v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table,
+                                                           T* kcache, T* vcache) {
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int p = pos[r];
+    float* row = qkv + (size_t)r * ld;
+    const bool has_kv = kcache != nullptr;
+    size_t slot = 0;
+    bool slot_ok = false;
+    if (has_kv && p >= 0 && p / g.page < g.max_blocks) {
+        const int pg = block_table[(size_t)seq[r] * g.max_blocks + p / g.page];
+        slot_ok = pg >= 0 && pg < g.num_pages;
+        slot = (size_t)pg * g.G * g.page + (p % g.page);           // + kv head * page
+    }
+    const float fp = (float)p;
+    const int hp = g.rot_dims / 2, nq = g.H * hp, nk = has_kv ? g.G * hp : 0;
+    for (int i = tid; i < nq + nk; i += 256) {
+        const bool isq = i < nq;
+        const int j = isq ? i : i - nq, head = j / hp, pr = j % hp;
+        int c0, c1;
+        hy_pair(g.rot_layout, pr, g.rot_dims, c0, c1);
+        float sn, cs;
+        sincosf(fp * kfreq[pr], &sn, &cs);
+        float* base = row + (isq ? 0 : koff) + head * g.dim;
+        const float u = base[c0], v = base[c1];
+        const float ru = u * cs - v * sn, rv = v * cs + u * sn;
+        if (isq) { base[c0] = ru; base[c1] = rv; }
+        else if (slot_ok) {
+            T* kd = kcache + (slot + (size_t)head * g.page) * g.dim;
+            kd[c0] = (T)ru; kd[c1] = (T)rv;
+        }
+    }
+    if (!has_kv || !slot_ok) return;
+    const int pass = g.dim - g.rot_dims;                             // key channels beyond the rotary span
+    for (int i = tid; i < g.G * pass; i += 256) {
+        const int head = i / pass, c = g.rot_dims + i % pass;
+        kcache[(slot + (size_t)head * g.page) * g.dim + c] = (T)row[koff + head * g.dim + c];
+    }
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int head = wave; head < g.G; head += 4) {
+        const float* v = row + voff + head * g.vdim;
+        T* vd = vcache + (slot + (size_t)head * g.page) * g.vdim;
+        float inv = 1.f;
+        if (v_norm) {
+            float ss = 0.f;
+            for (int c = lane; c < g.vdim; c += 64) ss = __builtin_fmaf(v[c], v[c], ss);
+            inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)g.vdim + eps);
+        }
+        if (vfreq) {
+            for (int m = lane; m < g.vdim / 2; m += 64) {
+                int c0, c1;
+                hy_pair(g.v_layout, m, g.vdim, c0, c1);
+                float sn, cs;
+                sincosf(fp * vfreq[m], &sn, &cs);
+                const float a = v[c0] * inv, b = v[c1] * inv;
+                vd[c0] = (T)(a * cs - b * sn); vd[c1] = (T)(b * cs + a * sn);
+            }
+        } else {
+            for (int c = lane; c < g.vdim; c += 64) vd[c] = (T)(v[c] * inv);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ attention over the paged cache, one wave per (row, head)
+constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
+
+template <typename T>
+__global__ __launch_bounds__(64) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+                                                          const int32_t* pos, const int32_t* seq, const int32_t* block_table,
+                                                          const T* kcache, const T* vcache, T* out) {
+    __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
+    __shared__ float p_s[64];
+    __shared__ long long row_s[64];
+    __shared__ float o_s[HY_MAX_VDIM];
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int p = pos[r], kvh = h / (g.H / g.G);
+    const int32_t* bt = block_table + (size_t)seq[r] * g.max_blocks;
+    for (int d = lane; d < g.dim; d += 64) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
+    __syncthreads();
+    const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
+    // running maximum m, denominator l and weighted value sum acc; the sink is a key of score 0 without a value: m = 0, l = 1 at the start
+    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+    float acc[HY_MAX_VDIM / 64];
+#pragma unroll
+    for (int i = 0; i < HY_MAX_VDIM / 64; ++i) acc[i] = 0.f;
+    for (int t0 = lo; t0 <= p; t0 += 64) {
+        const int kj = t0 + lane;
+        const bool valid = kj <= p;
+        float s = -INFINITY;
+        long long rowi = 0;
+        if (valid) {
+            const int pg = bt[kj / g.page];
+            rowi = ((long long)pg * g.G + kvh) * g.page + (kj % g.page);
+            const T* kp = kcache + rowi * g.dim;
+            float d0 = 0.f;
+            if (g.dim % 8 == 0) {
+                for (int d = 0; d < g.dim; d += 8) {
+                    float kv[8];
+                    hy_load8<T>(kp + d, kv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) d0 = __builtin_fmaf(q_s[d + i], kv[i], d0);
+                }
+            } else {
+                for (int d = 0; d < g.dim; ++d) d0 = __builtin_fmaf(q_s[d], (float)kp[d], d0);
+            }
+            s = d0 * scale;
+        }
+        const float mn = fmaxf(m, hy_wave_max(s));
+        const float pj = valid ? expf(s - mn) : 0.f;
+        const float corr = (mn == -INFINITY) ? 1.f : expf(m - mn);
+        l = l * corr + hy_wave_sum(pj);
+        m = mn;
+        __syncthreads();
+        p_s[lane] = pj; row_s[lane] = rowi;
+        __syncthreads();
+        const int nv = min(64, p - t0 + 1);
+#pragma unroll
+        for (int i = 0; i < HY_MAX_VDIM / 64; ++i) {
+            const int c = lane + 64 * i;
+            if (c >= g.vdim) break;
+            float a = acc[i] * corr;
+            for (int j = 0; j < nv; ++j) a = __builtin_fmaf(p_s[j], (float)vcache[row_s[j] * g.vdim + c], a);
+            acc[i] = a;
+        }
+    }
+    const float invl = l > 0.f ? 1.f / l : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < HY_MAX_VDIM / 64; ++i) { const int c = lane + 64 * i; if (c < g.vdim) o_s[c] = acc[i] * invl; }
+    __syncthreads();
+    T* od = out + ((size_t)r * g.H + h) * g.vdim;
+    if (vfreq) {     // turn the summed values back by the query's own position
+        const float fp = (float)p;
+        for (int mm = lane; mm < g.vdim / 2; mm += 64) {
+            int c0, c1;
+            hy_pair(g.v_layout, mm, g.vdim, c0, c1);
+            float sn, cs;
+            sincosf(fp * vfreq[mm], &sn, &cs);
+            const float a = o_s[c0], b = o_s[c1];
+            od[c0] = (T)(a * cs + b * sn); od[c1] = (T)(b * cs - a * sn);
+        }
+    } else {
+        for (int c = lane; c < g.vdim; c += 64) od[c] = (T)o_s[c];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ gated linear recurrence
+constexpr int SC_D = 32, SC_MAXDS = 8;
+enum { SCAN_HGRN2 = 0, SCAN_GLA = 1 };
+
+struct ScanParams {
+    const float* proj; int ld; int qo, ko, vo;     // fp32 projections [rows, ld]: q, k (GLA) or forget pre-activation (HGRN2), v at these columns
+    const float* z; int ldz;                        // GLA: decay pre-activation [rows, H * dim]
+    const void* lower; const void* fbias;           // HGRN2: lower bound and bias of the forget gate [H * dim], activation type
+    float tau, qscale;
+    int mode, H, dim, vdim;
+    const int32_t* row_start; const int32_t* slot; const int32_t* first_pos;
+    float* state;                                   // [slots, H, dim, vdim]
+    float* out;                                     // [rows, H * vdim]
+    int tok;                                        // tokens staged per pass
+};
+
+template <typename T>
+__global__ __launch_bounds__(512) void hy_scan_kernel(ScanParams p) {
+    extern __shared__ float hy_sm[];
+    const int DS = blockDim.x >> 6, dpad = DS * SC_D, SC_TOK = p.tok;
+    float* q_s = hy_sm;                          // [SC_TOK][dpad]
+    float* k_s = q_s + SC_TOK * dpad;
+    float* a_s = k_s + SC_TOK * dpad;
+    float* v_s = a_s + SC_TOK * dpad;            // [SC_TOK][64]
+    float* part_s = v_s + SC_TOK * 64;           // [SC_TOK][DS][64]
+    const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
+    const int tid = threadIdx.x, c = tid & 63, ds = tid >> 6;
+    const int r0 = p.row_start[sq], r1 = p.row_start[sq + 1];
+    const bool vok = v0 + c < p.vdim;
+    float* st = p.state + (((size_t)p.slot[sq] * p.H + h) * p.dim) * p.vdim + v0 + c;
+    float s[SC_D];
+    const bool fresh = p.first_pos[sq] == 0;
+#pragma unroll
+    for (int j = 0; j < SC_D; ++j) {
+        const int d = ds * SC_D + j;
+        s[j] = (!fresh && vok && d < p.dim) ? st[(size_t)d * p.vdim] : 0.f;
+    }
+    for (int t0 = r0; t0 < r1; t0 += SC_TOK) {
+        const int nt = min(SC_TOK, r1 - t0);
+        for (int i = tid; i < nt * dpad; i += blockDim.x) {
+            const int t = i / dpad, d = i % dpad;
+            float qv = 0.f, kv = 0.f, av = 1.f;
+            if (d < p.dim) {
+                const float* row = p.proj + (size_t)(t0 + t) * p.ld;
+                const int hd = h * p.dim + d;
+                if (p.mode == SCAN_HGRN2) {
+                    const float lw = (float)((const T*)p.lower)[hd];
+                    const float f = lw + (1.f - lw) * hy_sigmoid(row[p.ko + hd] + (float)((const T*)p.fbias)[hd]);
+                    qv = hy_silu(row[p.qo + hd]); av = f; kv = 1.f - f;
+                } else {
+                    const float zz = p.z[(size_t)(t0 + t) * p.ldz + hd];
+                    const float ls = fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)));       // log sigmoid(z)
+                    qv = row[p.qo + hd] * p.qscale; kv = row[p.ko + hd]; av = expf(ls / p.tau);
+                }
+            }
+            q_s[i] = qv; k_s[i] = kv; a_s[i] = av;
+        }
+        for (int i = tid; i < nt * 64; i += blockDim.x) {
+            const int t = i >> 6, cc = i & 63;
+            v_s[i] = (v0 + cc < p.vdim) ? p.proj[(size_t)(t0 + t) * p.ld + p.vo + h * p.vdim + v0 + cc] : 0.f;
+        }
+        __syncthreads();
+        for (int t = 0; t < nt; ++t) {
+            const float vt = v_s[t * 64 + c];
+            const float* qq = q_s + t * dpad + ds * SC_D;
+            const float* kk = k_s + t * dpad + ds * SC_D;
+            const float* aa = a_s + t * dpad + ds * SC_D;
+            float o = 0.f;
+#pragma unroll
+            for (int j = 0; j < SC_D; ++j) {
+                s[j] = __builtin_fmaf(aa[j], s[j], kk[j] * vt);
+                o = __builtin_fmaf(s[j], qq[j], o);
+            }
+            part_s[(t * DS + ds) * 64 + c] = o;
+        }
+        __syncthreads();
+        for (int i = tid; i < nt * 64; i += blockDim.x) {
+            const int t = i >> 6, cc = i & 63;
+            if (v0 + cc >= p.vdim) continue;
+            float o = 0.f;
+            for (int k = 0; k < DS; ++k) o += part_s[(t * DS + k) * 64 + cc];
+            p.out[(size_t)(t0 + t) * p.H * p.vdim + h * p.vdim + v0 + cc] = o;
+        }
+    }
+    if (vok) {
+#pragma unroll
+        for (int j = 0; j < SC_D; ++j) {
+            const int d = ds * SC_D + j;
+            if (d < p.dim) st[(size_t)d * p.vdim] = s[j];
+        }
+    }
+}
+
+// per-head RMS norm over vdim with a plain weight shared by the heads, optional silu gate: one wave per (row, head)
+template <typename T>
+__global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out) {
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* src = o + ((size_t)r * H + h) * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64) ss = __builtin_fmaf(src[c], src[c], ss);
+    const float inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)vdim + eps);
+    for (int c = lane; c < vdim; c += 64) {
+        float v = src[c] * inv * (float)w[c];
+        if (gate) v *= hy_silu(gate[(size_t)r * ldg + goff + h * vdim + c]);
+        out[((size_t)r * H + h) * vdim + c] = (T)v;
+    }
+}
+
+int hy_geom_ok(const AttnGeom& g) {
+    MI355_CHECK_ARG(g.H > 0 && g.G > 0 && g.H % g.G == 0, "hybrid attention: heads=%d kv_heads=%d", g.H, g.G);
+    MI355_CHECK_ARG(g.dim > 0 && g.dim <= HY_MAX_DIM, "hybrid attention: head size %d (<= %d)", g.dim, HY_MAX_DIM);
+    MI355_CHECK_ARG(g.vdim > 0 && g.vdim % 2 == 0 && g.vdim <= HY_MAX_VDIM, "hybrid attention: value size %d (even, <= %d)", g.vdim, HY_MAX_VDIM);
+    MI355_CHECK_ARG(g.rot_dims >= 0 && g.rot_dims <= g.dim && g.rot_dims % 2 == 0, "hybrid attention: rotary span %d of %d", g.rot_dims, g.dim);
+    MI355_CHECK_ARG(g.page > 0 && g.max_blocks > 0 && g.num_pages > 0, "hybrid attention: page=%d max_blocks=%d pages=%d", g.page, g.max_blocks, g.num_pages);
+    return MI355_OK;
+}
+
+#define HY_DISPATCH(dt, ...)                                                          \
+    do {                                                                              \
+        if ((dt) == MI355_ACT_BF16) { using T = bf16; __VA_ARGS__; }                  \
+        else if ((dt) == MI355_ACT_F32) { using T = float; __VA_ARGS__; }             \
+        else { mi355_set_error("hybrid op: act_dtype=%d (bf16 or fp32)", (int)(dt)); return MI355_ERR_ARG; } \
+    } while (0)
+
+} // namespace
+
+extern "C" int mi355_hy_embed(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float* out, int32_t act_dtype,
+                              mi355_stream_t stream) {
+    MI355_CHECK_ARG(ids && table && out && rows > 0 && W > 0 && vocab > 0, "hy_embed: rows=%d W=%d", rows, W);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_embed_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, ids, (const T*)table, W, vocab, out));
+    MI355_CHECK_LAUNCH("hy_embed_kernel");
+    return MI355_OK;
+}
+
+// x [*, W] fp32 stream; a, b [*, W] fp32 branch outputs (either may be null); rows: null, or `n` source rows to gather (x is then read only).
+// h1 / h2 [n, W] of act_dtype: x / rms(x) * (weight_offset + w).  w2 / h2 may be null.
+extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, float mult, const int32_t* rows, int32_t n, int32_t W,
+                                      const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
+                                      mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && n > 0 && W > 0 && (!h1 || w1) && (!h2 || w2), "hy_residual_norm: n=%d W=%d", n, W);
+    MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_residual_norm: W=%d too wide for one block", W);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_residual_norm_kernel<T>, dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
+                                              (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
+    MI355_CHECK_LAUNCH("hy_residual_norm_kernel");
+    return MI355_OK;
+}
+
+// geom: {H, G, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages}.  qkv fp32 [rows, ld]: q heads at column 0 (rotated in
+// place), k heads at koff, v heads at voff.  kcache [pages, G, page, dim], vcache [pages, G, page, vdim] of act_dtype; null kcache: queries only
+// (a layer that reads another layer's cache).  kfreq [rot_dims / 2], vfreq [vdim / 2] fp32 angular steps (vfreq null: values are not rotated).
+extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
+                                  int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
+                                  void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(qkv && geom && pos && seq && rows > 0, "hy_attn_prep: null argument");
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    if (int e = hy_geom_ok(g)) return e;
+    MI355_CHECK_ARG((g.rot_dims == 0 || kfreq) && (!kcache || (vcache && block_table)), "hy_attn_prep: missing table or cache");
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_prep_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, qkv, ld, koff, voff, g, kfreq, vfreq,
+                                              v_norm, eps, pos, seq, block_table, (T*)kcache, (T*)vcache));
+    MI355_CHECK_LAUNCH("hy_attn_prep_kernel");
+    return MI355_OK;
+}
+
+// out [rows, H * vdim] of act_dtype.  chunk > 0: row at position i sees keys j <= i of its own block of `chunk` positions; 0: all j <= i.
+// sink: one is added to the softmax denominator.  vfreq non-null: the head output is turned back by the row's position.
+extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+                                  const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
+                                  const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    if (int e = hy_geom_ok(g)) return e;
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
+                                              pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out));
+    MI355_CHECK_LAUNCH("hy_attn_rows_kernel");
+    return MI355_OK;
+}
+
+// mode 0 (HGRN2): q = silu(proj q), f = lower + (1 - lower) sigmoid(proj k + fbias), a = f, k = 1 - f.
+// mode 1 (GLA):   q = proj q * qscale, k = proj k, a = sigmoid(z)^(1 / tau).
+// Sequence s owns rows row_start[s] .. row_start[s + 1] - 1 in order, continues the state in slot[s] (starts from zero when first_pos[s] == 0)
+// and leaves the new state there.  out fp32 [rows, H * vdim].
+extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
+                             const void* lower, const void* fbias, float tau, float qscale, int32_t H, int32_t dim, int32_t vdim,
+                             const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,
+                             int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(proj && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_scan: bad argument");
+    MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : (mode == SCAN_GLA && z && tau > 0.f), "hy_scan: mode %d lacks its gate inputs", mode);
+    const int DS = (dim + SC_D - 1) / SC_D;
+    MI355_CHECK_ARG(DS <= SC_MAXDS, "hy_scan: key size %d > %d", dim, SC_MAXDS * SC_D);
+    const int tok = DS > 4 ? 8 : 16;       // keeps the staging buffers under 64 KiB of LDS at every key size
+    ScanParams p{proj, ld, qo, ko, vo, z, ldz, lower, fbias, tau, qscale, mode, H, dim, vdim, row_start, slot, first_pos, state, out, tok};
+    const size_t lds = (size_t)(3 * tok * DS * SC_D + tok * 64 + tok * DS * 64) * 4;
+    const dim3 grid(nseq, H, (vdim + 63) / 64);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_scan_kernel<T>, grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
+    MI355_CHECK_LAUNCH("hy_scan_kernel");
+    return MI355_OK;
+}
+
+extern "C" int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
+                                  int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(o && w && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps, gate, ldg,
+                                              goff, (T*)out));
+    MI355_CHECK_LAUNCH("hy_head_norm_kernel");
+    return MI355_OK;
+}

@@ -1,0 +1,161 @@
+"""The hybrid decoder family: a stack of parallel-residual layers  x <- x + m * (mixer(norm1 x) + mlp(norm2 x))  over an fp32 residual
+stream, every layer with its own mixer (mixers.PagedChunkAttention or mixers.GatedLinearRecurrence) and an optional gated MLP, a final
+norm, the output head and an optional tanh soft cap of the logits.  Norm weights are stored as offsets from one.
+
+``HybridConfig.from_json`` reads the family's config.json (keys: architecture, vocab, width, residual_mult, logit_softcap, norm.eps and
+layers[i].{type, mixer, mlp}); ``HybridModel`` holds the device weights (checkpoint tensors embed, l<i>.norm1/2, l<i>.mix.*, l<i>.mlp.*,
+final.norm, head) and runs one ragged step against the cache tensors an engine allocated from ``cache_layout()``.
+
+Nufalorn is the member of the family registered here: chunk-masked sink attention with unit-normed, rotated values and shared-KV
+layers, HGRN2 and GLA recurrences, relu-gated MLPs."""
+import json
+import os
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Union
+
+import torch
+
+from . import hybrid_ops as hops
+from .mixers import AttentionSpec, GatedLinearRecurrence, GatedMLP, PagedChunkAttention, RecurrenceSpec, RotarySpec, StepBatch
+
+
+@dataclass
+class HybridLayerSpec:
+    kind: str                                        # "attention" | "hgrn2" | "gla"
+    mixer: Union[AttentionSpec, RecurrenceSpec]
+    ff: Optional[int] = None                         # None: the layer has no MLP
+    mlp_act: str = "relu"
+
+
+@dataclass
+class HybridConfig:
+    name: str
+    vocab: int
+    width: int
+    layers: List[HybridLayerSpec]
+    eps: float = 1e-5
+    residual_mult: float = 1.0
+    logit_softcap: float = 0.0
+    norm_offset: float = 1.0                         # stored norm weights are offsets from this value
+
+    @staticmethod
+    def from_json(cfg: dict) -> "HybridConfig":
+        """The Nufalorn reading of config.json: attention layers have the softmax sink, unit-normed values and values rotated in the key
+        layout (interleaved pairs); MLPs are relu-gated; norm weights are stored around zero."""
+        layers = []
+        for i, L in enumerate(cfg["layers"]):
+            kind, mx, mlp = L["type"], L["mixer"], L.get("mlp")
+            if kind == "attention":
+                rot = mx.get("rot")
+                rs = RotarySpec(int(rot["dims"]), float(rot["base"]), "interleaved") if rot and int(rot.get("dims", 0)) else None
+                mask = mx.get("mask") or {}
+                spec = AttentionSpec(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx["vdim"]),
+                                     scale=float(mx["scale"]), rot=rs, chunk=int(mask.get("size", 0) or 0), sink=True, value_norm=True,
+                                     value_rot=rs is not None, value_layout="interleaved",
+                                     kv_from=None if mx.get("kv_from") is None else int(mx["kv_from"]))
+            elif kind in ("hgrn2", "gla"):
+                spec = RecurrenceSpec(kind, heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx["vdim"]), tau=float(mx.get("tau", 1.0)))
+            else:
+                raise NotImplementedError(f"layer {i}: mixer type {kind!r}")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise NotImplementedError(f"layer {i}: mlp kind {mlp.get('kind')!r}")
+            layers.append(HybridLayerSpec(kind, spec, None if mlp is None else int(mlp["ff"]), "relu"))
+        for i, L in enumerate(layers):
+            src = getattr(L.mixer, "kv_from", None)
+            if src is not None:
+                o = layers[src].mixer if 0 <= src < i else None
+                if not isinstance(o, AttentionSpec) or o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (L.mixer.kv_heads, L.mixer.dim, L.mixer.vdim):
+                    raise ValueError(f"layer {i}: kv_from {src} must name an earlier attention layer with its own keys and values of the same shape")
+        return HybridConfig(name=str(cfg.get("architecture", "hybrid")), vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers,
+                            eps=float(cfg["norm"]["eps"]), residual_mult=float(cfg.get("residual_mult", 1.0)),
+                            logit_softcap=float(cfg.get("logit_softcap") or 0.0))
+
+
+class HybridModel:
+    """Device weights + the step function.  dtype: torch.bfloat16 (16-bit weights and activations, fp32 accumulation and fp32 for everything
+    the family keeps in 32-bit) or torch.float32 (everything in true fp32)."""
+
+    def __init__(self, cfg: HybridConfig, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device, page: int = 64):
+        hops.act_code(dtype)
+        self.cfg, self.dtype, self.device, self.page = cfg, dtype, torch.device(device), page
+
+        def get(name):
+            if name not in tensors:
+                raise KeyError(f"checkpoint has no tensor {name!r}")
+            return tensors[name].to(device=self.device, dtype=dtype).contiguous()
+
+        def sub(prefix, names):
+            return {n: get(prefix + n) for n in names}
+
+        self.embed = get("embed")
+        self.head = get("head")
+        self.final_norm = get("final.norm")
+        if self.embed.shape != (cfg.vocab, cfg.width) or self.head.shape != (cfg.vocab, cfg.width):
+            raise ValueError(f"embed {tuple(self.embed.shape)} / head {tuple(self.head.shape)} against vocab {cfg.vocab} width {cfg.width}")
+        self.layers = []
+        for i, L in enumerate(cfg.layers):
+            p = f"l{i}."
+            if L.kind == "attention":
+                names = ["q", "o"] + (["k", "v"] if L.mixer.kv_from is None else [])
+                mixer = PagedChunkAttention(L.mixer, sub(p + "mix.", names), cfg.eps, page, self.device)
+            elif L.kind == "hgrn2":
+                mixer = GatedLinearRecurrence(L.mixer, sub(p + "mix.", ["q", "f", "f.b", "lower", "v", "norm", "o"]), cfg.eps)
+            else:
+                mixer = GatedLinearRecurrence(L.mixer, sub(p + "mix.", ["q", "k", "v", "g", "a1", "a2", "a2.b", "norm", "o"]), cfg.eps)
+            mlp = None
+            if L.ff is not None:
+                mlp = GatedMLP(get(p + "mlp.gate"), get(p + "mlp.up"), get(p + "mlp.down"), L.mlp_act)
+            self.layers.append((L, mixer, mlp, get(p + "norm1"), get(p + "norm2") if mlp is not None else None))
+        self.has_state = any(L.kind != "attention" for L in cfg.layers)
+
+    # ---- what an engine has to allocate
+    def cache_layout(self):
+        """Per layer: ("kv", K page shape, V page shape) | ("kv_from", layer) | ("state", per-slot shape)."""
+        out = []
+        for L, mixer, _, _, _ in self.layers:
+            if L.kind == "attention":
+                out.append(("kv",) + mixer.cache_shapes() if mixer.owns_cache else ("kv_from", L.mixer.kv_from))
+            else:
+                out.append(("state", mixer.state_shape()))
+        return out
+
+    def alloc_cache(self, num_pages: int, num_slots: int):
+        """Cache tensors for `num_pages` pages and `num_slots` state slots: per layer (kcache, vcache) or a state tensor."""
+        caches = []
+        for ent in self.cache_layout():
+            if ent[0] == "kv":
+                caches.append((torch.zeros(num_pages, *ent[1], dtype=self.dtype, device=self.device),
+                               torch.zeros(num_pages, *ent[2], dtype=self.dtype, device=self.device)))
+            elif ent[0] == "kv_from":
+                caches.append(caches[ent[1]])
+            else:
+                caches.append(torch.zeros(num_slots, *ent[1], dtype=torch.float32, device=self.device))
+        return caches
+
+    # ---- one step
+    def forward(self, batch: StepBatch, caches, collect: Optional[list] = None) -> torch.Tensor:
+        """fp32 logits [len(batch.want), vocab] of the wanted rows; the caches of every row's sequence are advanced.  collect: receives
+        the residual stream after every layer (debugging / tests; costs one extra norm launch per layer)."""
+        cfg = self.cfg
+        x = hops.embed(batch.tokens, self.embed)
+        a = b = None
+        for (L, mixer, mlp, n1, n2), cache in zip(self.layers, caches):
+            h1, h2 = hops.residual_norm(x, a, b, cfg.residual_mult, n1, n2, cfg.eps, weight_offset=cfg.norm_offset)
+            if collect is not None and a is not None:
+                collect.append(x.clone())
+            a = mixer.forward(h1, batch, *cache) if L.kind == "attention" else mixer.forward(h1, batch, cache)
+            b = mlp.forward(h2) if mlp is not None else None
+        if collect is not None:
+            hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset)
+            collect.append(x.clone())
+            a = b = None
+        hf, _ = hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want)
+        return hops.dense_linear(hf, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
+
+
+def load_hybrid_checkpoint(path: str, dtype: torch.dtype, device, page: int = 64) -> HybridModel:
+    """A folder with config.json and *.safetensors of the family -> HybridModel on `device`."""
+    from .loader import _Shards
+    cfg = HybridConfig.from_json(json.load(open(os.path.join(path, "config.json"))))
+    sh = _Shards(path)
+    return HybridModel(cfg, {k: sh.get(k) for k in sh.map}, dtype, device, page)

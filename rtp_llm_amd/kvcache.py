@@ -75,3 +75,87 @@ def read_tokens(kv_base: torch.Tensor, scale_base: Optional[torch.Tensor], block
     if scale_base is None:
         return K, V, None, None
     return _flip(K), _flip(V), scale_base[blk, 0, :, off], scale_base[blk, 1, :, off]
+
+
+# --------------------------------------------------------------------------- pool management for the serving engine
+class PagePool:
+    """Free list of KV pages shared by all layers (page i of every layer belongs to the same owner).  A fresh pool hands out pages
+    0, 1, 2, ...; a page that came back is the next one handed out."""
+
+    def __init__(self, num_pages: int):
+        if num_pages <= 0:
+            raise ValueError(f"PagePool: {num_pages} pages")
+        self.num_pages = num_pages
+        self._free = list(range(num_pages - 1, -1, -1))
+
+    @property
+    def free(self) -> int:
+        return len(self._free)
+
+    def take(self, n: int):
+        if n > len(self._free):
+            raise MemoryError(f"PagePool: {n} pages wanted, {len(self._free)} free of {self.num_pages}")
+        out = [self._free.pop() for _ in range(n)]
+        return out
+
+    def give(self, pages):
+        for p in pages:
+            if not 0 <= p < self.num_pages or p in self._free:
+                raise ValueError(f"PagePool: page {p} is not out")
+            self._free.append(p)
+
+
+class SlotPool(PagePool):
+    """Fixed-size slots of per-sequence state (the recurrent layers' fp32 states): one per live sequence."""
+
+
+class SequenceCache:
+    """What one live sequence holds: its pages (in position order), its state slot and the number of tokens already run."""
+
+    def __init__(self, slot: int):
+        self.pages, self.slot, self.length = [], slot, 0
+
+
+class CacheManager:
+    """Pages and state slots of the live sequences of one engine.  `page` tokens per page; a sequence gets pages as it grows and gives
+    everything back on release.  reserve: pages promised to admitted sequences for tokens they have not run yet (generation)."""
+
+    def __init__(self, num_pages: int, page: int, num_slots: int):
+        self.page = page
+        self.pages, self.slots = PagePool(num_pages), SlotPool(num_slots)
+        self.live = {}
+        self._promised = {}
+
+    def pages_for(self, tokens: int) -> int:
+        return (tokens + self.page - 1) // self.page
+
+    def can_admit(self, total_tokens: int) -> bool:
+        return self.slots.free > 0 and self.pages.free - sum(self._promised.values()) >= self.pages_for(total_tokens)
+
+    def admit(self, sid, reserve_tokens: int = 0) -> SequenceCache:
+        if sid in self.live:
+            raise KeyError(f"sequence {sid!r} is already live")
+        if self.slots.free == 0:
+            raise MemoryError(f"no state slot free for {sid!r} ({self.slots.num_pages} live sequences at most)")
+        sc = SequenceCache(self.slots.take(1)[0])
+        self.live[sid] = sc
+        self._promised[sid] = self.pages_for(reserve_tokens)
+        return sc
+
+    def grow(self, sid, new_tokens: int) -> SequenceCache:
+        """Make room for `new_tokens` more tokens of a live sequence (its length moves when the step has run: advance())."""
+        sc = self.live[sid]
+        need = self.pages_for(sc.length + new_tokens) - len(sc.pages)
+        if need > 0:
+            sc.pages += self.pages.take(need)
+            self._promised[sid] = max(0, self._promised[sid] - need)
+        return sc
+
+    def advance(self, sid, new_tokens: int):
+        self.live[sid].length += new_tokens
+
+    def release(self, sid):
+        sc = self.live.pop(sid)
+        self._promised.pop(sid, None)
+        self.pages.give(sc.pages)
+        self.slots.give([sc.slot])
