@@ -211,7 +211,15 @@ def main():
     ap.add_argument("--debug-set", default="", help="debug only: 'idx=val,...' forwarded to mi355_debug_set (kernel A/B switches)")
     ap.add_argument("--attn-ps", type=int, default=0, help="debug only (tuning build): tokens per attention partition instead of the planner's choice")
     ap.add_argument("--prefetch", type=int, default=None, help="weight-prefetch mask (mi355_decoder_set_weight_prefetch); default: the engine's")
+    ap.add_argument("--hybrid", action="store_true", help="instead of the default workload: prefill / decode throughput and kernel rooflines of the hybrid "
+                    "decoder family beside the Qwen2 engine at equal sizes (rtp_llm_amd/bench_hybrid.py); 1 GPU")
+    ap.add_argument("--hybrid-sizes", default="", help="--hybrid: comma-separated subset of w1024,w2048,w4096")
+    ap.add_argument("--hybrid-prompt", type=int, default=2048)
+    ap.add_argument("--hybrid-batch", type=int, default=16)
     args = ap.parse_args()
+    if args.hybrid:
+        from rtp_llm_amd import bench_hybrid
+        sys.exit(bench_hybrid.run(args))
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # plain `python bench.py --gpus N` (no launcher): this process becomes the launcher of N ranks

@@ -41,6 +41,9 @@ class ServingEngine:
         self.cache = CacheManager(num_pages, self.page, max_seqs)
         self.tensors = model.alloc_cache(num_pages, max_seqs)
         self.max_step_tokens = max_step_tokens
+        # decode-only steps (one token per entry, its logits wanted) replay a captured HIP graph per (sequences, block-table width)
+        self.use_graphs = False
+        self._graphs = {}
         self.waiting: List[Request] = []
         self.running: List[Request] = []
 
@@ -48,7 +51,15 @@ class ServingEngine:
     def build_batch(self, entries: Sequence[Tuple[object, Sequence[int], Sequence[int]]]) -> StepBatch:
         """entries: (sequence id, its next tokens, indices among them whose logits are wanted).  Admits new sequences and takes pages."""
         tokens, pos, seq, row_start, slot, first, want, tables = [], [], [], [0], [], [], [], []
-        seen = set()
+        seen, admitted = set(), []
+        try:
+            return self._build(entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted)
+        except Exception:
+            for sid in admitted:                      # a step that cannot run leaves no half-admitted sequence behind
+                self.cache.release(sid)
+            raise
+
+    def _build(self, entries, tokens, pos, seq, row_start, slot, first, want, tables, seen, admitted):
         for sid, toks, wants in entries:
             if sid in seen:
                 raise ValueError(f"sequence {sid!r} appears twice in one step")
@@ -57,6 +68,7 @@ class ServingEngine:
                 raise ValueError(f"sequence {sid!r}: an entry without tokens")
             if sid not in self.cache.live:
                 self.cache.admit(sid)
+                admitted.append(sid)
             sc = self.cache.grow(sid, len(toks))
             s = len(slot)
             base = len(tokens)
@@ -84,10 +96,32 @@ class ServingEngine:
         if not entries:
             return None
         batch = self.build_batch(entries)
-        logits = self.model.forward(batch, self.tensors, collect)
+        if self.use_graphs and collect is None and all(len(t) == 1 and list(w) == [0] for _, t, w in entries):
+            logits = self._replay_decode(batch)
+        else:
+            logits = self.model.forward(batch, self.tensors, collect)
         for sid, toks, _ in entries:
             self.cache.advance(sid, len(toks))
         return logits if batch.want.numel() else None
+
+    def _replay_decode(self, batch: StepBatch) -> torch.Tensor:
+        """The decode step as a graph: captured once per shape over static input tensors (capture runs nothing, so the recurrent states
+        move only on replay), then fed by copies into those tensors."""
+        fields = ("tokens", "pos", "seq", "row_start", "slot", "first_pos", "block_table", "want")
+        key = (batch.slot.numel(), batch.block_table.shape[1])
+        ent = self._graphs.get(key)
+        if ent is None:
+            static = StepBatch(*[getattr(batch, f).clone() for f in fields])
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                out = self.model.forward(static, self.tensors)
+            ent = self._graphs[key] = (g, static, out)
+        g, static, out = ent
+        for f in fields:
+            getattr(static, f).copy_(getattr(batch, f), non_blocking=True)
+        g.replay()
+        return out.clone()
 
     def release(self, sid):
         self.cache.release(sid)
