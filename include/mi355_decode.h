@@ -717,6 +717,9 @@ int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const
 int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
                        const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
                        const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+                        const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0, const int32_t* tile_n,
+                        int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
                   const void* lower, const void* fbias, float tau, float qscale, int32_t H, int32_t dim, int32_t vdim,
                   const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,

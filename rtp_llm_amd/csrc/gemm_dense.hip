@@ -5,7 +5,8 @@
 // decays, shared-KV attention) loads its tensors as they are.  Three kernels, all with fp32 accumulation and an fp32 epilogue:
 //   * tile kernel, bf16:  64 x 128 block tile, 4 waves of 32 x 64, K staged through LDS 64 at a time, MFMA 16x16x32;
 //   * tile kernel, fp32:  64 x 64 block tile, 4 x 4 register micro-tiles, true fp32 FMAs (no reduced-precision matrix mode);
-//   * row kernel (M <= 16): one wave per output column streams its weight row once, 16-byte loads, wave reduction at the end.
+//   * skinny kernel, bf16, 2 <= M <= 16: one block per 16 outputs, its waves split K, MFMA fragments loaded straight from memory;
+//   * row kernel (M = 1; fp32 up to M = 16): a wave per output column streams its weight row once, 16-byte loads, wave reduction at the end.
 // Epilogues: bias, gated activation act(gate) * up (weight rows grouped [32 gate | 32 up], so one lane holds both), tanh soft cap.
 // Output is fp32 or the activation type.  A result row depends only on its own input row: the k order of the accumulation is fixed by
 // the kernel, never by M or by the row's place in the batch.
@@ -237,46 +238,134 @@ __device__ __forceinline__ float dn_wave_sum(float v) {
     return v;
 }
 
-// One wave per output: a plain column n, or under `gated` one channel c (gate row and up row).  MR rows of x per pass.
-template <typename T, int MR>
+// One wave per NC outputs: plain columns, or under GATED channels (a gate row and an up row each).  MR rows of x per pass: every 16-byte
+// piece of x is loaded once per wave and meets NC (2 NC) weight pieces, so the wave streams its weight rows with few loads of x between.
+template <typename T, int MR, int NC, bool GATED>
 __global__ __launch_bounds__(256) void dense_rows_kernel(DenseParams p, int mbase) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int o = blockIdx.x * 4 + wave;
-    const int nout = p.gated ? p.N / 2 : p.N;
-    if (o >= nout) return;
-    const int n0 = p.gated ? (o >> 5) * 64 + (o & 31) : o;
+    const int o0 = (blockIdx.x * 4 + wave) * NC;
+    const int nout = GATED ? p.N / 2 : p.N;
+    if (o0 >= nout) return;
     const T* X = (const T*)p.x;
-    const T* W0 = (const T*)p.w + (size_t)n0 * p.K;
-    const T* W1 = W0 + (size_t)32 * p.K;
-    const int rows = min(MR, p.M - mbase);
-    float a0[MR], a1[MR];
+    const T* W0[NC];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) { a0[m] = 0.f; a1[m] = 0.f; }
+    for (int c = 0; c < NC; ++c) {
+        const int o = min(o0 + c, nout - 1);                       // a column past the end repeats the last one and is not stored
+        W0[c] = (const T*)p.w + (size_t)(GATED ? (o >> 5) * 64 + (o & 31) : o) * p.K;
+    }
+    const int rows = min(MR, p.M - mbase);
+    float a0[MR][NC], a1[GATED ? MR : 1][NC];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) { a0[m][c] = 0.f; if (GATED) a1[m][c] = 0.f; }
     for (int k = lane * 8; k < p.K; k += 64 * 8) {
-        float w0[8], w1[8], xv[8];
-        DnVec<T>::load(W0 + k, p.K - k, p.vec, w0);
-        if (p.gated) DnVec<T>::load(W1 + k, p.K - k, p.vec, w1);
+        float w0[NC][8], w1[GATED ? NC : 1][8], xv[8];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            DnVec<T>::load(W0[c] + k, p.K - k, p.vec, w0[c]);
+            if (GATED) DnVec<T>::load(W0[c] + (size_t)32 * p.K + k, p.K - k, p.vec, w1[c]);
+        }
 #pragma unroll
         for (int m = 0; m < MR; ++m) {
             if (m >= rows) break;
             DnVec<T>::load(X + (size_t)(mbase + m) * p.ldx + k, p.K - k, p.vec, xv);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) a0[m] = __builtin_fmaf(xv[i], w0[i], a0[m]);
-            if (p.gated) {
+            for (int c = 0; c < NC; ++c) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) a1[m] = __builtin_fmaf(xv[i], w1[i], a1[m]);
+                for (int i = 0; i < 8; ++i) a0[m][c] = __builtin_fmaf(xv[i], w0[c][i], a0[m][c]);
+                if (GATED) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a1[m][c] = __builtin_fmaf(xv[i], w1[c][i], a1[m][c]);
+                }
             }
         }
     }
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         if (m >= rows) break;
-        float g = dn_wave_sum(a0[m]);
-        float u = p.gated ? dn_wave_sum(a1[m]) : 0.f;
-        if (lane != 0) continue;
-        if (p.bias) { g += dn_ld((const T*)p.bias + n0); if (p.gated) u += dn_ld((const T*)p.bias + n0 + 32); }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            float g = dn_wave_sum(a0[m][c]);
+            float u = GATED ? dn_wave_sum(a1[m][c]) : 0.f;
+            const int o = o0 + c;
+            if (lane != 0 || o >= nout) continue;
+            const int n0 = GATED ? (o >> 5) * 64 + (o & 31) : o;
+            if (p.bias) { g += dn_ld((const T*)p.bias + n0); if (GATED) u += dn_ld((const T*)p.bias + n0 + 32); }
+            g = dn_act(g, p.act);
+            dn_store<T>(p, mbase + m, o, GATED ? g * u : g);
+        }
+    }
+}
+
+template <typename T, bool GATED>
+void launch_rows(const DenseParams& p, hipStream_t st) {
+    const int nout = GATED ? p.N / 2 : p.N;
+    for (int mb = 0; mb < p.M; mb += 16) {
+        const int r = p.M - mb;
+        // few rows: one output per wave keeps the most waves streaming; more rows: several outputs per wave share the loads of x
+        if (r <= 2)      hipLaunchKernelGGL((dense_rows_kernel<T, 2, 1, GATED>), dim3((nout + 3) / 4), dim3(256), 0, st, p, mb);
+        else if (r <= 4) hipLaunchKernelGGL((dense_rows_kernel<T, 4, 2, GATED>), dim3((nout + 7) / 8), dim3(256), 0, st, p, mb);
+        else if (r <= 8) hipLaunchKernelGGL((dense_rows_kernel<T, 8, GATED ? 2 : 4, GATED>), dim3((nout + (GATED ? 7 : 15)) / (GATED ? 8 : 16)), dim3(256), 0, st, p, mb);
+        else             hipLaunchKernelGGL((dense_rows_kernel<T, 16, GATED ? 2 : 4, GATED>), dim3((nout + (GATED ? 7 : 15)) / (GATED ? 8 : 16)), dim3(256), 0, st, p, mb);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ skinny kernel (bf16, M <= 16)
+// One block per 16 outputs; its NW waves split K in interleaved steps of 32 and each wave runs MFMA 16x16x32 with the (up to) 16 rows of x as
+// the A operand and 16 weight rows as B, both fragments loaded straight from memory (8 consecutive k per lane, no LDS staging).  The weight
+// stream is read once whatever M is; the waves' partial tiles are summed through LDS.  Under GATED a tile is 16 channels: their gate rows and
+// their up rows share the A fragments.
+template <bool GATED>
+__global__ __launch_bounds__(512) void dense_skinny_bf16_kernel(DenseParams p, int mbase) {
+    __shared__ f32x4 red[8][2][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, NW = blockDim.x >> 6;
+    const int nout = GATED ? p.N / 2 : p.N;
+    const int r = lane & 15, kq = (lane >> 4) * 8;
+    const int o = min((int)blockIdx.x * 16 + r, nout - 1);
+    const int n = GATED ? (o >> 5) * 64 + (o & 31) : o;
+    const bf16* wg = (const bf16*)p.w + (size_t)n * p.K + kq;
+    const bf16* wu = wg + (size_t)32 * p.K;
+    const bf16* xr = (const bf16*)p.x + (size_t)min(mbase + r, p.M - 1) * p.ldx + kq;
+    f32x4 ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+    const bf16x8 zero = {};
+    const int stride = NW * 32;
+    for (int k0 = wave * 32; k0 < p.K; k0 += 4 * stride) {
+        bf16x8 a[4], b[4], c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int k = k0 + u * stride;
+            const bool ok = k + kq < p.K;
+            a[u] = ok ? *(const bf16x8*)(xr + k) : zero;
+            b[u] = ok ? *(const bf16x8*)(wg + k) : zero;
+            if (GATED) c[u] = ok ? *(const bf16x8*)(wu + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            ag = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u], ag, 0, 0, 0);
+            if (GATED) au = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], c[u], au, 0, 0, 0);
+        }
+    }
+    red[wave][0][lane] = ag;
+    if (GATED) red[wave][1][lane] = au;
+    __syncthreads();
+    if (wave != 0) return;
+    for (int w = 1; w < NW; ++w) {
+        ag += red[w][0][lane];
+        if (GATED) au += red[w][1][lane];
+    }
+    // C fragment: lane holds output (lane & 15), rows 4 * (lane >> 4) + e
+    const int oc = blockIdx.x * 16 + r;
+    if (oc >= nout) return;
+    const int nb = GATED ? (oc >> 5) * 64 + (oc & 31) : oc;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int row = mbase + (lane >> 4) * 4 + e;
+        if (row >= p.M) continue;
+        float g = ag[e], u = au[e];
+        if (p.bias) { g += dn_ld((const bf16*)p.bias + nb); if (GATED) u += dn_ld((const bf16*)p.bias + nb + 32); }
         g = dn_act(g, p.act);
-        dn_store<T>(p, mbase + m, o, p.gated ? g * u : g);
+        dn_store<bf16>(p, row, oc, GATED ? g * u : g);
     }
 }
 
@@ -302,21 +391,17 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
     (void)es;
     hipStream_t st = (hipStream_t)stream;
+    if (bf && M > 1 && M <= 16 && p.vec) {
+        const int tiles = ((gated ? N / 2 : N) + 15) / 16;
+        const int nw = (tiles >= 1024 || K < 1024) ? 4 : 8;        // narrow outputs: more waves per tile keep the memory system busy
+        if (gated) hipLaunchKernelGGL(dense_skinny_bf16_kernel<true>, dim3(tiles), dim3(64 * nw), 0, st, p, 0);
+        else       hipLaunchKernelGGL(dense_skinny_bf16_kernel<false>, dim3(tiles), dim3(64 * nw), 0, st, p, 0);
+        MI355_CHECK_LAUNCH("dense_skinny_bf16_kernel");
+        return MI355_OK;
+    }
     if (M <= 16) {
-        const int nout = gated ? N / 2 : N;
-        const dim3 grid((nout + 3) / 4);
-        for (int mb = 0; mb < M; mb += 8) {
-            const int r = M - mb;
-            if (bf) {
-                if (r <= 2)      hipLaunchKernelGGL((dense_rows_kernel<bf16, 2>), grid, dim3(256), 0, st, p, mb);
-                else if (r <= 4) hipLaunchKernelGGL((dense_rows_kernel<bf16, 4>), grid, dim3(256), 0, st, p, mb);
-                else             hipLaunchKernelGGL((dense_rows_kernel<bf16, 8>), grid, dim3(256), 0, st, p, mb);
-            } else {
-                if (r <= 2)      hipLaunchKernelGGL((dense_rows_kernel<float, 2>), grid, dim3(256), 0, st, p, mb);
-                else if (r <= 4) hipLaunchKernelGGL((dense_rows_kernel<float, 4>), grid, dim3(256), 0, st, p, mb);
-                else             hipLaunchKernelGGL((dense_rows_kernel<float, 8>), grid, dim3(256), 0, st, p, mb);
-            }
-        }
+        if (bf) { if (gated) launch_rows<bf16, true>(p, st); else launch_rows<bf16, false>(p, st); }
+        else    { if (gated) launch_rows<float, true>(p, st); else launch_rows<float, false>(p, st); }
         MI355_CHECK_LAUNCH("dense_rows_kernel");
         return MI355_OK;
     }

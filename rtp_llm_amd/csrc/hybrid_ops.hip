@@ -148,44 +148,62 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
     }
 }
 
-// ------------------------------------------------------------------------------------------------ attention over the paged cache, one wave per (row, head)
+// ------------------------------------------------------------------------------------------------ attention over the paged cache
 constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
 
+// Four waves per (row, head): wave w takes the 64-key tiles w, w + 4, ... of the row's visible range with its own running maximum,
+// denominator and value sum; the four are merged at the end.  Inside a tile a lane scores one key (its whole q . k), the tile's weights and
+// page rows then travel by lane broadcast (uniform loop index -> v_readlane), and a lane accumulates its own value channels over the keys.
+__device__ __forceinline__ float hy_lane_f(float v, int j) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), j)); }
+
 template <typename T>
-__global__ __launch_bounds__(64) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
-                                                          const int32_t* pos, const int32_t* seq, const int32_t* block_table,
-                                                          const T* kcache, const T* vcache, T* out) {
+__global__ __launch_bounds__(256) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+                                                           const int32_t* pos, const int32_t* seq, const int32_t* block_table,
+                                                           const T* kcache, const T* vcache, T* out) {
+    constexpr int NV = HY_MAX_VDIM / 64;
     __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
-    __shared__ float p_s[64];
-    __shared__ long long row_s[64];
+    __shared__ float m_s[4], l_s[4];
+    __shared__ float acc_s[4][HY_MAX_VDIM];
+    __shared__ float part_s[4][64][8];
     __shared__ float o_s[HY_MAX_VDIM];
-    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int p = pos[r], kvh = h / (g.H / g.G);
+    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int p = __builtin_amdgcn_readfirstlane(pos[r]), kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r] * g.max_blocks;
-    for (int d = lane; d < g.dim; d += 64) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
+    for (int d = tid; d < g.dim; d += 256) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
     __syncthreads();
     const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
-    // running maximum m, denominator l and weighted value sum acc; the sink is a key of score 0 without a value: m = 0, l = 1 at the start
-    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
-    float acc[HY_MAX_VDIM / 64];
+    // the sink is a key of score 0 that carries no value: wave 0 starts from m = 0, l = 1
+    float m = (sink && wave == 0) ? 0.f : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
+    float acc[NV], facc[8];
 #pragma unroll
-    for (int i = 0; i < HY_MAX_VDIM / 64; ++i) acc[i] = 0.f;
-    for (int t0 = lo; t0 <= p; t0 += 64) {
+    for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) facc[i] = 0.f;
+    const bool fast = g.vdim % 8 == 0;
+    const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 256: KPI >= 2)
+    const int grp = lane / LPK, cl = (lane % LPK) * 8;
+    const bool gok = grp < KPI;
+    for (int t0 = lo + wave * 64; t0 <= p; t0 += 256) {
         const int kj = t0 + lane;
         const bool valid = kj <= p;
         float s = -INFINITY;
-        long long rowi = 0;
+        int rowi = 0;                                              // row of the key inside the cache tensors: (page * G + kv head) * page size + offset
         if (valid) {
-            const int pg = bt[kj / g.page];
-            rowi = ((long long)pg * g.G + kvh) * g.page + (kj % g.page);
-            const T* kp = kcache + rowi * g.dim;
+            rowi = (bt[kj / g.page] * g.G + kvh) * g.page + (kj % g.page);
+            const T* kp = kcache + (size_t)rowi * g.dim;
             float d0 = 0.f;
             if (g.dim % 8 == 0) {
-                for (int d = 0; d < g.dim; d += 8) {
-                    float kv[8];
-                    hy_load8<T>(kp + d, kv);
+                for (int d = 0; d < g.dim; d += 64) {              // eight 16-byte pieces of the key row in flight
+                    float kv[8][8];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) d0 = __builtin_fmaf(q_s[d + i], kv[i], d0);
+                    for (int u = 0; u < 8; ++u)
+                        if (d + 8 * u < g.dim) hy_load8<T>(kp + d + 8 * u, kv[u]);
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        if (d + 8 * u < g.dim) {
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) d0 = __builtin_fmaf(q_s[d + 8 * u + i], kv[u][i], d0);
+                        }
                 }
             } else {
                 for (int d = 0; d < g.dim; ++d) d0 = __builtin_fmaf(q_s[d], (float)kp[d], d0);
@@ -194,45 +212,244 @@ __global__ __launch_bounds__(64) void hy_attn_rows_kernel(const float* q, int ld
         }
         const float mn = fmaxf(m, hy_wave_max(s));
         const float pj = valid ? expf(s - mn) : 0.f;
-        const float corr = (mn == -INFINITY) ? 1.f : expf(m - mn);
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
         l = l * corr + hy_wave_sum(pj);
         m = mn;
-        __syncthreads();
-        p_s[lane] = pj; row_s[lane] = rowi;
-        __syncthreads();
         const int nv = min(64, p - t0 + 1);
+        if (fast) {
+            // LPK lanes share one key's value row (8 channels = 16 bytes each), so one load instruction covers KPI keys
 #pragma unroll
-        for (int i = 0; i < HY_MAX_VDIM / 64; ++i) {
-            const int c = lane + 64 * i;
-            if (c >= g.vdim) break;
-            float a = acc[i] * corr;
-            for (int j = 0; j < nv; ++j) a = __builtin_fmaf(p_s[j], (float)vcache[row_s[j] * g.vdim + c], a);
-            acc[i] = a;
+            for (int i = 0; i < 8; ++i) facc[i] *= corr;
+            for (int j = 0; j < nv; j += 4 * KPI) {
+                float pw[4], vv[4][8];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int kk = j + u * KPI + grp;
+                    const bool ok = gok && kk < nv;
+                    const float pk = __shfl(pj, kk & 63, 64);
+                    const int rk = __shfl(rowi, kk & 63, 64);
+                    pw[u] = ok ? pk : 0.f;
+                    if (ok) hy_load8<T>(vcache + (size_t)rk * g.vdim + cl, vv[u]);
+                    else {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) vv[u][i] = 0.f;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) facc[i] = __builtin_fmaf(pw[u], vv[u][i], facc[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane + 64 * i;
+                if (64 * i >= g.vdim) break;
+                const bool cok = c < g.vdim;
+                float a = acc[i] * corr;
+                for (int j = 0; j < nv; ++j) {
+                    const float pw = hy_lane_f(pj, j);
+                    const size_t vr = (size_t)__builtin_amdgcn_readlane(rowi, j) * g.vdim;
+                    a = __builtin_fmaf(pw, cok ? (float)vcache[vr + c] : 0.f, a);
+                }
+                acc[i] = a;
+            }
         }
     }
-    const float invl = l > 0.f ? 1.f / l : 0.f;
-    __syncthreads();
+    if (fast) {       // sum the KPI partial rows of this wave into acc_s[wave]
 #pragma unroll
-    for (int i = 0; i < HY_MAX_VDIM / 64; ++i) { const int c = lane + 64 * i; if (c < g.vdim) o_s[c] = acc[i] * invl; }
+        for (int i = 0; i < 8; ++i) part_s[wave][lane][i] = facc[i];
+        __syncthreads();
+        for (int c = lane; c < g.vdim; c += 64) {
+            float a = 0.f;
+            for (int k = 0; k < KPI; ++k) a += part_s[wave][k * LPK + (c >> 3)][c & 7];
+            acc_s[wave][c] = a;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) { const int c = lane + 64 * i; if (c < g.vdim) acc_s[wave][c] = acc[i]; }
+    }
+    if (lane == 0) { m_s[wave] = m; l_s[wave] = l; }
+    __syncthreads();
+    const float mm = fmaxf(fmaxf(m_s[0], m_s[1]), fmaxf(m_s[2], m_s[3]));
+    float w4[4], lt = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { w4[w] = (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm); lt = __builtin_fmaf(l_s[w], w4[w], lt); }
+    const float invl = lt > 0.f ? 1.f / lt : 0.f;
+    for (int c = tid; c < g.vdim; c += 256)
+        o_s[c] = (acc_s[0][c] * w4[0] + acc_s[1][c] * w4[1] + acc_s[2][c] * w4[2] + acc_s[3][c] * w4[3]) * invl;
     __syncthreads();
     T* od = out + ((size_t)r * g.H + h) * g.vdim;
     if (vfreq) {     // turn the summed values back by the query's own position
         const float fp = (float)p;
-        for (int mm = lane; mm < g.vdim / 2; mm += 64) {
+        for (int mi = tid; mi < g.vdim / 2; mi += 256) {
             int c0, c1;
-            hy_pair(g.v_layout, mm, g.vdim, c0, c1);
+            hy_pair(g.v_layout, mi, g.vdim, c0, c1);
             float sn, cs;
-            sincosf(fp * vfreq[mm], &sn, &cs);
+            sincosf(fp * vfreq[mi], &sn, &cs);
             const float a = o_s[c0], b = o_s[c1];
             od[c0] = (T)(a * cs + b * sn); od[c1] = (T)(b * cs - a * sn);
         }
     } else {
-        for (int c = lane; c < g.vdim; c += 64) od[c] = (T)o_s[c];
+        for (int c = tid; c < g.vdim; c += 256) od[c] = (T)o_s[c];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ attention for prompt portions: MFMA tiles (bf16 cache)
+// One wave per (tile of up to 16 consecutive rows of one sequence, head).  Keys go by 32: S = Q K^T with v_mfma_f32_16x16x32_bf16 (K fragments
+// straight from the cache: 8 consecutive channels per lane), mask and online softmax on the fp32 accumulator fragments, then O += P V with P
+// passed through LDS into the A layout and the 32 value rows transposed through LDS into the B layout.  Scores and weights stay 32-bit: the
+// fp32 queries (scaled) and the fp32 weights enter the matrix unit as an exact sum of two bf16 terms (high part + remainder), the cached
+// keys and values are bf16 as stored, every accumulation is fp32.
+__device__ __forceinline__ void hy_split_bf16(float x, bf16& hi, bf16& lo) { hi = (bf16)x; lo = (bf16)(x - (float)hi); }
+__device__ __forceinline__ float hy_max16(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float hy_sum16(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
+
+__global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+                                                           const int32_t* pos, const int32_t* seq, const int32_t* block_table,
+                                                           const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
+                                                           bf16* out) {
+    __shared__ __attribute__((aligned(16))) bf16 Ph[16 * AT_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Pl[16 * AT_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Vt[HY_MAX_VDIM * AT_LD];
+    const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, lr = lane & 15, lq = lane >> 4;
+    const int r0 = tile_row0[tile], n = tile_n[tile];
+    const int p0 = pos[r0], kvh = h / (g.H / g.G);
+    const int32_t* bt = block_table + (size_t)seq[r0] * g.max_blocks;
+    const int DK = g.dim / 32, NCB = g.vdim / 16, VP = g.vdim / 8;
+    bf16x8 qh[8], ql[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        if (ks >= DK) break;
+        const float* qp = q + (size_t)(r0 + min(lr, n - 1)) * ldq + h * g.dim + ks * 32 + lq * 8;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { bf16 a, b; hy_split_bf16(qp[i] * scale, a, b); qh[ks][i] = a; ql[ks][i] = b; }
+    }
+    float m[4], l[4];
+    f32x4 o[16];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { m[e] = sink ? 0.f : -INFINITY; l[e] = (sink && lr == 0) ? 1.f : 0.f; }   // l: per-lane share of the row's denominator
+#pragma unroll
+    for (int cb = 0; cb < 16; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int plast = p0 + n - 1;
+    const int kstart = (chunk > 0 ? (p0 / chunk) * chunk : 0) & ~31;
+    for (int t0 = kstart; t0 <= plast; t0 += 32) {
+        f32x4 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int kc = min(t0 + kb * 16 + lr, plast);
+            const bf16* kp = kcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.dim + lq * 8;
+            bf16x8 kf[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) if (ks < DK) kf[ks] = *(const bf16x8*)(kp + ks * 32);
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+                if (ks < DK) {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[ks], kf[ks], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[ks], kf[ks], acc, 0, 0, 0);
+                }
+            s[kb] = acc;
+        }
+        // the 32 value rows, transposed: Vt[channel][key]
+        for (int i = lane; i < 32 * VP; i += 64) {
+            const int key = i / VP, c8 = (i % VP) * 8;
+            const int kc = min(t0 + key, plast);
+            const u32x4 raw = *(const u32x4*)(vcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.vdim + c8);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *(uint16_t*)&Vt[(c8 + 2 * j) * AT_LD + key] = (uint16_t)(raw[j] & 0xFFFFu);
+                *(uint16_t*)&Vt[(c8 + 2 * j + 1) * AT_LD + key] = (uint16_t)(raw[j] >> 16);
+            }
+        }
+        // mask, running maximum, weights; fragment element e is row 4 lq + e, the lane's key columns are kb * 16 + lr
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = lq * 4 + e, rpos = p0 + row;
+            const int rlo = chunk > 0 ? (rpos / chunk) * chunk : 0;
+            float sv[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const int kpos = t0 + kb * 16 + lr;
+                sv[kb] = (row < n && kpos <= rpos && kpos >= rlo) ? s[kb][e] : -INFINITY;
+            }
+            const float mn = fmaxf(m[e], hy_max16(fmaxf(sv[0], sv[1])));
+            float pw[2] = {0.f, 0.f}, corr = 1.f;
+            if (mn != -INFINITY) {
+                corr = (m[e] == -INFINITY) ? 0.f : expf(m[e] - mn);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) pw[kb] = (sv[kb] == -INFINITY) ? 0.f : expf(sv[kb] - mn);
+            }
+            l[e] = l[e] * corr + pw[0] + pw[1];
+            m[e] = mn;
+#pragma unroll
+            for (int cb = 0; cb < 16; ++cb) if (cb < NCB) o[cb][e] *= corr;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                bf16 a, b;
+                hy_split_bf16(pw[kb], a, b);
+                Ph[row * AT_LD + kb * 16 + lr] = a; Pl[row * AT_LD + kb * 16 + lr] = b;
+            }
+        }
+        __syncthreads();
+        const bf16x8 ph = *(const bf16x8*)&Ph[lr * AT_LD + lq * 8], pl = *(const bf16x8*)&Pl[lr * AT_LD + lq * 8];
+#pragma unroll
+        for (int cb = 0; cb < 16; ++cb)
+            if (cb < NCB) {
+                const bf16x8 vf = *(const bf16x8*)&Vt[(cb * 16 + lr) * AT_LD + lq * 8];
+                o[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, vf, o[cb], 0, 0, 0);
+                o[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, vf, o[cb], 0, 0, 0);
+            }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int row = lq * 4 + e;
+        const float lt = hy_sum16(l[e]);
+        const float inv = lt > 0.f ? 1.f / lt : 0.f;
+        const float fp = (float)(p0 + row);
+        bf16* od = out + ((size_t)(r0 + row) * g.H + h) * g.vdim;
+#pragma unroll
+        for (int cb = 0; cb < 16; ++cb) {
+            if (cb >= NCB) break;
+            const int c = cb * 16 + lr;
+            float v = o[cb][e] * inv;
+            if (vfreq) {          // turn back by the row's position; the partner channel sits in the next lane (interleaved) or NCB / 2 fragments away (halves)
+                float other, sn, cs;
+                bool first;
+                int mi;
+                if (g.v_layout == 0) { other = __shfl_xor(v, 1, 64); first = (c & 1) == 0; mi = c >> 1; }
+                else {
+                    const int half = NCB / 2;
+                    first = cb < half; mi = first ? c : c - g.vdim / 2;
+                    float t = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) if (k == (first ? cb + half : cb - half)) t = o[k][e] * inv;
+                    other = t;
+                }
+                sincosf(fp * vfreq[mi], &sn, &cs);
+                v = first ? (v * cs + other * sn) : (v * cs - other * sn);
+            }
+            if (row < n) od[c] = (bf16)v;
+        }
     }
 }
 
 // ------------------------------------------------------------------------------------------------ gated linear recurrence
-constexpr int SC_D = 32, SC_MAXDS = 8;
+// Block = 64 value columns x DS groups of RD key rows: thread (c, ds) keeps S[ds * RD .. + RD - 1][c] in registers.  Tokens are staged `tok`
+// at a time: all threads compute the gates of the staged tokens once into LDS, then every thread walks the tokens in order (its RD rows:
+// decay, rank-one update, partial q . S), and the DS partial outputs per token are summed from LDS.  Short RD keeps the dependent chain per
+// token short; the walk itself is the sequential part of the recurrence.
 enum { SCAN_HGRN2 = 0, SCAN_GLA = 1 };
 
 struct ScanParams {
@@ -247,29 +464,29 @@ struct ScanParams {
     int tok;                                        // tokens staged per pass
 };
 
-template <typename T>
-__global__ __launch_bounds__(512) void hy_scan_kernel(ScanParams p) {
-    extern __shared__ float hy_sm[];
-    const int DS = blockDim.x >> 6, dpad = DS * SC_D, SC_TOK = p.tok;
-    float* q_s = hy_sm;                          // [SC_TOK][dpad]
-    float* k_s = q_s + SC_TOK * dpad;
-    float* a_s = k_s + SC_TOK * dpad;
-    float* v_s = a_s + SC_TOK * dpad;            // [SC_TOK][64]
-    float* part_s = v_s + SC_TOK * 64;           // [SC_TOK][DS][64]
+template <typename T, int RD>
+__global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
+    extern __shared__ __attribute__((aligned(16))) float hy_sm[];
+    const int DS = blockDim.x >> 6, dpad = DS * RD, TOK = p.tok;
+    float* q_s = hy_sm;                          // [TOK][dpad]
+    float* k_s = q_s + TOK * dpad;
+    float* a_s = k_s + TOK * dpad;
+    float* v_s = a_s + TOK * dpad;               // [TOK][64]
+    float* part_s = v_s + TOK * 64;              // [TOK][DS][64]
     const int sq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * 64;
     const int tid = threadIdx.x, c = tid & 63, ds = tid >> 6;
     const int r0 = p.row_start[sq], r1 = p.row_start[sq + 1];
     const bool vok = v0 + c < p.vdim;
     float* st = p.state + (((size_t)p.slot[sq] * p.H + h) * p.dim) * p.vdim + v0 + c;
-    float s[SC_D];
+    float s[RD];
     const bool fresh = p.first_pos[sq] == 0;
 #pragma unroll
-    for (int j = 0; j < SC_D; ++j) {
-        const int d = ds * SC_D + j;
+    for (int j = 0; j < RD; ++j) {
+        const int d = ds * RD + j;
         s[j] = (!fresh && vok && d < p.dim) ? st[(size_t)d * p.vdim] : 0.f;
     }
-    for (int t0 = r0; t0 < r1; t0 += SC_TOK) {
-        const int nt = min(SC_TOK, r1 - t0);
+    for (int t0 = r0; t0 < r1; t0 += TOK) {
+        const int nt = min(TOK, r1 - t0);
         for (int i = tid; i < nt * dpad; i += blockDim.x) {
             const int t = i / dpad, d = i % dpad;
             float qv = 0.f, kv = 0.f, av = 1.f;
@@ -295,16 +512,21 @@ __global__ __launch_bounds__(512) void hy_scan_kernel(ScanParams p) {
         __syncthreads();
         for (int t = 0; t < nt; ++t) {
             const float vt = v_s[t * 64 + c];
-            const float* qq = q_s + t * dpad + ds * SC_D;
-            const float* kk = k_s + t * dpad + ds * SC_D;
-            const float* aa = a_s + t * dpad + ds * SC_D;
-            float o = 0.f;
+            const f32x4* qq = (const f32x4*)(q_s + t * dpad + ds * RD);
+            const f32x4* kk = (const f32x4*)(k_s + t * dpad + ds * RD);
+            const f32x4* aa = (const f32x4*)(a_s + t * dpad + ds * RD);
+            float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < SC_D; ++j) {
-                s[j] = __builtin_fmaf(aa[j], s[j], kk[j] * vt);
-                o = __builtin_fmaf(s[j], qq[j], o);
+            for (int j4 = 0; j4 < RD / 4; ++j4) {
+                const f32x4 a4 = aa[j4], k4 = kk[j4], q4 = qq[j4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int j = j4 * 4 + e;
+                    s[j] = __builtin_fmaf(a4[e], s[j], k4[e] * vt);
+                    o[e] = __builtin_fmaf(s[j], q4[e], o[e]);
+                }
             }
-            part_s[(t * DS + ds) * 64 + c] = o;
+            part_s[(t * DS + ds) * 64 + c] = (o[0] + o[1]) + (o[2] + o[3]);
         }
         __syncthreads();
         for (int i = tid; i < nt * 64; i += blockDim.x) {
@@ -317,8 +539,8 @@ __global__ __launch_bounds__(512) void hy_scan_kernel(ScanParams p) {
     }
     if (vok) {
 #pragma unroll
-        for (int j = 0; j < SC_D; ++j) {
-            const int d = ds * SC_D + j;
+        for (int j = 0; j < RD; ++j) {
+            const int d = ds * RD + j;
             if (d < p.dim) st[(size_t)d * p.vdim] = s[j];
         }
     }
@@ -345,6 +567,7 @@ int hy_geom_ok(const AttnGeom& g) {
     MI355_CHECK_ARG(g.vdim > 0 && g.vdim % 2 == 0 && g.vdim <= HY_MAX_VDIM, "hybrid attention: value size %d (even, <= %d)", g.vdim, HY_MAX_VDIM);
     MI355_CHECK_ARG(g.rot_dims >= 0 && g.rot_dims <= g.dim && g.rot_dims % 2 == 0, "hybrid attention: rotary span %d of %d", g.rot_dims, g.dim);
     MI355_CHECK_ARG(g.page > 0 && g.max_blocks > 0 && g.num_pages > 0, "hybrid attention: page=%d max_blocks=%d pages=%d", g.page, g.max_blocks, g.num_pages);
+    MI355_CHECK_ARG((long long)g.num_pages * g.G * g.page < (1ll << 31), "hybrid attention: %d pages x %d heads x %d tokens overflow a 32-bit row index", g.num_pages, g.G, g.page);
     return MI355_OK;
 }
 
@@ -402,9 +625,28 @@ extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, cons
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
     if (int e = hy_geom_ok(g)) return e;
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(256), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
                                               pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out));
     MI355_CHECK_LAUNCH("hy_attn_rows_kernel");
+    return MI355_OK;
+}
+
+// The same attention for prompt portions (bf16 cache): tile t covers rows tile_row0[t] .. + tile_n[t] - 1 (<= 16, consecutive positions of one
+// sequence).  Needs dim % 32 == 0 and vdim % 16 == 0 (% 32 under the halves layout), both <= 256: MI355_ERR_UNSUPPORTED otherwise.
+extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+                                   const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0,
+                                   const int32_t* tile_n, int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype,
+                                   mi355_stream_t stream) {
+    MI355_CHECK_ARG(q && geom && pos && seq && block_table && tile_row0 && tile_n && kcache && vcache && out && tiles > 0 && chunk >= 0, "hy_attn_tiles: bad argument");
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    if (int e = hy_geom_ok(g)) return e;
+    if (act_dtype != MI355_ACT_BF16 || g.dim % 32 || g.dim > 256 || g.vdim % 16 || g.vdim > 256 || (vfreq && g.v_layout != 0 && g.vdim % 32)) {
+        mi355_set_error("hy_attn_tiles: bf16, dim %% 32 == 0, vdim %% 16 == 0 only (dim=%d vdim=%d dtype=%d)", g.dim, g.vdim, act_dtype);
+        return MI355_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(hy_attn_tiles_kernel, dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq, block_table,
+                       tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
+    MI355_CHECK_LAUNCH("hy_attn_tiles_kernel");
     return MI355_OK;
 }
 
@@ -418,13 +660,18 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
                              int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(proj && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_scan: bad argument");
     MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : (mode == SCAN_GLA && z && tau > 0.f), "hy_scan: mode %d lacks its gate inputs", mode);
-    const int DS = (dim + SC_D - 1) / SC_D;
-    MI355_CHECK_ARG(DS <= SC_MAXDS, "hy_scan: key size %d > %d", dim, SC_MAXDS * SC_D);
-    const int tok = DS > 4 ? 8 : 16;       // keeps the staging buffers under 64 KiB of LDS at every key size
+    MI355_CHECK_ARG(dim <= 512, "hy_scan: key size %d > 512", dim);
+    const int RD = dim <= 128 ? 8 : dim <= 256 ? 16 : 32;       // rows per thread: at most 16 groups of RD rows (1024 threads)
+    const int DS = (dim + RD - 1) / RD;
+    int tok = 16;                                                // staged tokens: keep the LDS buffers under 60 KiB
+    auto lds_of = [&](int t) { return (size_t)(3 * t * DS * RD + t * 64 + t * DS * 64) * 4; };
+    while (tok > 1 && lds_of(tok) > 60 * 1024) tok >>= 1;
     ScanParams p{proj, ld, qo, ko, vo, z, ldz, lower, fbias, tau, qscale, mode, H, dim, vdim, row_start, slot, first_pos, state, out, tok};
-    const size_t lds = (size_t)(3 * tok * DS * SC_D + tok * 64 + tok * DS * 64) * 4;
+    const size_t lds = lds_of(tok);
     const dim3 grid(nseq, H, (vdim + 63) / 64);
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_scan_kernel<T>, grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
+    if (RD == 8)       HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 8>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
+    else if (RD == 16) HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 16>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
+    else               HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_scan_kernel<T, 32>), grid, dim3(64 * DS), lds, (hipStream_t)stream, p));
     MI355_CHECK_LAUNCH("hy_scan_kernel");
     return MI355_OK;
 }

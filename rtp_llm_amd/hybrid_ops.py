@@ -158,6 +158,26 @@ def attn_rows(q: torch.Tensor, scale: float, geom, chunk: int, sink: bool, vfreq
     return out
 
 
+def attn_tiles_supported(dtype: torch.dtype, dim: int, vdim: int, value_rot: bool, v_layout: int) -> bool:
+    """Shapes the MFMA kernel for prompt portions takes (attn_rows serves every other)."""
+    return dtype == torch.bfloat16 and dim % 32 == 0 and dim <= 256 and vdim % 16 == 0 and vdim <= 256 and not (value_rot and v_layout and vdim % 32)
+
+
+def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: bool, vfreq, pos, seq, block_table, tile_row0, tile_n, kcache, vcache,
+               heads: int, vdim: int):
+    """attn_rows for prompt portions on the matrix cores: tile t = rows tile_row0[t] .. + tile_n[t] - 1 (at most 16 consecutive rows of one
+    sequence); every row of the batch must lie in exactly one tile."""
+    _dev(q, torch.float32, "attn_tiles.q"); _dev(tile_row0, torch.int32, "attn_tiles.tile_row0"); _dev(tile_n, torch.int32, "attn_tiles.tile_n")
+    T = q.shape[0]
+    out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_tiles(q.data_ptr(), _rows(q, "attn_tiles.q"), float(scale), geom, int(chunk), 1 if sink else 0, _p(vfreq),
+                                                            pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), tile_row0.data_ptr(), tile_n.data_ptr(),
+                                                            tile_row0.numel(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
+                                                            act_code(kcache.dtype), _stream()), "hy_attn_tiles")
+    return out
+
+
 def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[torch.Tensor], lower, fbias, tau: float, qscale: float,
          heads: int, dim: int, vdim: int, row_start, slot, first_pos, state: torch.Tensor, act: torch.dtype) -> torch.Tensor:
     """Gated linear recurrence over the rows of every sequence, continuing (and leaving) the fp32 state of its slot -> fp32 [T, heads * vdim]."""

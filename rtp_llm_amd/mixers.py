@@ -64,6 +64,8 @@ class StepBatch:
     first_pos: torch.Tensor
     block_table: torch.Tensor
     want: torch.Tensor                   # rows whose logits are computed
+    tile_row0: Optional[torch.Tensor] = None   # tiles of at most 16 consecutive rows of one sequence covering every row: first row ...
+    tile_n: Optional[torch.Tensor] = None      # ... and row count (the matrix-core attention for prompt portions works on them)
 
 
 def rotary_steps(n_pairs: int, span: int, base: float, device) -> torch.Tensor:
@@ -87,6 +89,7 @@ class PagedChunkAttention:
         self.kfreq = rotary_steps(rot.dims // 2, rot.dims, rot.base, device) if rot and rot.dims else None
         self.vfreq = rotary_steps(s.vdim // 2, s.vdim, rot.base, device) if s.value_rot and rot else None
         self._geom = None
+        self.use_tiles = True
 
     def cache_shapes(self):
         """(K page tensor shape, V page tensor shape) without the leading page count."""
@@ -110,7 +113,14 @@ class PagedChunkAttention:
         write = self.owns_cache
         hops.attn_prep(qkv, self.koff, self.voff, geom, self.kfreq, self.vfreq, s.value_norm, self.eps, batch.pos, batch.seq, batch.block_table,
                        kcache if write else None, vcache if write else None)
-        o = hops.attn_rows(qkv, s.scale, geom, s.chunk, s.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim)
+        T = qkv.shape[0]
+        # prompt portions (tiles mostly full) go to the matrix-core kernel, decode rows to the one that spreads a row's keys over four waves
+        if (self.use_tiles and batch.tile_row0 is not None and batch.tile_row0.numel() * 4 <= T
+                and hops.attn_tiles_supported(kcache.dtype, s.dim, s.vdim, self.vfreq is not None, hops.LAYOUTS[s.value_layout])):
+            o = hops.attn_tiles(qkv, s.scale, geom, s.chunk, s.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n,
+                                kcache, vcache, s.heads, s.vdim)
+        else:
+            o = hops.attn_rows(qkv, s.scale, geom, s.chunk, s.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim)
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
 

@@ -88,7 +88,12 @@ class ServingEngine:
         for i, t in enumerate(tables):
             bt[i, : len(t)] = torch.tensor(t, dtype=torch.int32)
         i32 = lambda v: torch.tensor(v, dtype=torch.int32).to(self.device, non_blocking=True)
-        return StepBatch(i32(tokens), i32(pos), i32(seq), i32(row_start), i32(slot), i32(first), bt.to(self.device, non_blocking=True), i32(want))
+        t0, tn = [], []
+        for a, b in zip(row_start[:-1], row_start[1:]):           # tiles of at most 16 consecutive rows of one sequence
+            t0 += list(range(a, b, 16))
+            tn += [min(16, b - r) for r in range(a, b, 16)]
+        return StepBatch(i32(tokens), i32(pos), i32(seq), i32(row_start), i32(slot), i32(first), bt.to(self.device, non_blocking=True), i32(want),
+                         i32(t0), i32(tn))
 
     def run_step(self, entries, collect: Optional[list] = None) -> Optional[torch.Tensor]:
         """Run the entries as one batch; -> fp32 logits [wanted rows, vocab] in the order of the entries and their wants (None if none)."""
@@ -107,7 +112,7 @@ class ServingEngine:
     def _replay_decode(self, batch: StepBatch) -> torch.Tensor:
         """The decode step as a graph: captured once per shape over static input tensors (capture runs nothing, so the recurrent states
         move only on replay), then fed by copies into those tensors."""
-        fields = ("tokens", "pos", "seq", "row_start", "slot", "first_pos", "block_table", "want")
+        fields = ("tokens", "pos", "seq", "row_start", "slot", "first_pos", "block_table", "want", "tile_row0", "tile_n")
         key = (batch.slot.numel(), batch.block_table.shape[1])
         ent = self._graphs.get(key)
         if ent is None:

@@ -360,3 +360,47 @@ def test_graph_replayed_decode_steps_match_eager_and_oracle():
     for j, k in enumerate(("a", "b", "c")):
         close(out[j:j + 1], ref[k][at[k]:at[k] + 1], 3e-4)
     assert len(eng._graphs) == 2
+
+
+@pytest.mark.parametrize("dim,vdim,heads,kv_heads,chunk,layout", [(32, 16, 2, 1, 40, "interleaved"), (64, 48, 4, 2, 0, "interleaved"),
+                                                                   (128, 128, 4, 1, 100, "interleaved"), (96, 64, 3, 3, 33, "halves"),
+                                                                   (256, 256, 2, 2, 64, "interleaved")])
+def test_matrix_core_attention_for_portions_equals_row_kernel(dim, vdim, heads, kv_heads, chunk, layout):
+    """Both attention kernels over the same bf16 pages: ragged portions of three sequences that start inside pages and mask blocks, with
+    tiles of every fill (1 .. 16 rows), scattered pages, a sink and rotated values."""
+    from rtp_llm_amd import hybrid_ops as hops
+    from rtp_llm_amd.mixers import rotary_steps
+    g = torch.Generator(device=DEV).manual_seed(dim + vdim)
+    page, num_pages, width = 64, 24, 8
+    starts, counts = [0, 70, 250], [45, 130, 17]                       # first position and row count of each sequence's portion
+    tables = torch.randperm(num_pages, generator=torch.Generator().manual_seed(1), dtype=torch.int32)[:3 * width].reshape(3, width)
+    pos, seq, t0, tn, row = [], [], [], [], 0
+    for s_, (a, n) in enumerate(zip(starts, counts)):
+        pos += list(range(a, a + n)); seq += [s_] * n
+        t0 += list(range(row, row + n, 16)); tn += [min(16, n - r) for r in range(0, n, 16)]
+        row += n
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    kc = torch.randn(num_pages, kv_heads, page, dim, device=DEV, generator=g).bfloat16()
+    vc = torch.randn(num_pages, kv_heads, page, vdim, device=DEV, generator=g).bfloat16()
+    q = torch.randn(row, heads * dim, device=DEV, generator=g)
+    geom = hops.attn_geometry(heads, kv_heads, dim, vdim, dim, 0, hops.LAYOUTS[layout], page, width, num_pages)
+    vf = rotary_steps(vdim // 2, vdim, 1e4, DEV)
+    assert hops.attn_tiles_supported(torch.bfloat16, dim, vdim, True, hops.LAYOUTS[layout])
+    for sink, vfreq in ((True, vf), (False, None)):
+        a = hops.attn_rows(q, dim ** -0.5, geom, chunk, sink, vfreq, i32(pos), i32(seq), tables.to(DEV), kc, vc, heads, vdim)
+        b = hops.attn_tiles(q, dim ** -0.5, geom, chunk, sink, vfreq, i32(pos), i32(seq), tables.to(DEV), i32(t0), i32(tn), kc, vc, heads, vdim)
+        err = (a.float() - b.float()).abs()
+        assert float(err.max()) <= 2e-2 and float(err.mean()) < 1e-3, f"kernels differ: max {float(err.max())} mean {float(err.mean())}"
+
+
+def test_bf16_dominant_key_through_matrix_core_attention():
+    """The mask edges again in bfloat16, where prompt portions run on the matrix cores: the asker's logits with the beacon just inside and just
+    outside its block must each match the plain implementation (they differ from one another by far more than bf16 rounding)."""
+    for beacon, asker in ((64, 127), (63, 127), (127, 127 + 64), (0, 60)):
+        cfg, w = _beacon_model(64, dim=32, rot=16, vdim=32)
+        t = [3 + (i % 30) for i in range(asker + 1)]
+        t[beacon], t[asker] = 1, 2
+        ref = U.oracle_logits(cfg, w, t)[asker]
+        eng = engine(cfg, w, torch.bfloat16)
+        got = eng.run_step([("w", t, [asker])])[0].double().cpu()
+        assert float((got - ref).abs().max()) < 0.05 * float(ref.abs().max()) + 0.05
