@@ -73,9 +73,27 @@ def hybrid_weights(cfg, dev, seed=0):
     return w
 
 
-def timed(fn, reps=5, warm=2):
+def timed(fn, reps=5, warm=2, graph=False):
+    """Seconds per call.  graph: the calls are captured into one HIP graph and the replay is timed, so the figure is the kernels' own
+    time and not the host's launch path (what a graph-replayed step pays)."""
     for _ in range(warm):
         fn()
+    if graph:
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(reps):
+                fn()
+        inner, fn, reps = reps, g.replay, 3
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * inner) * 1e-3
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
@@ -149,6 +167,7 @@ def kernel_table(s, dev, prompt):
     """Time the kernels of both families at this size; roofline time = max(bytes / HBM, flops / peak of the unit that does them)."""
     from . import hybrid_ops as hops, ops, quant
     rows = []
+    timed_k = lambda fn: timed(fn, reps=10, warm=2, graph=True)
     g = torch.Generator(device=dev).manual_seed(3)
     bf = lambda *sh: torch.randn(*sh, device=dev, generator=g).bfloat16()
     W, H, G, hd, ff = s["width"], s["heads"], s["kv"], s["hd"], s["ff"]
@@ -162,25 +181,25 @@ def kernel_table(s, dev, prompt):
     for M_ in (prompt, 8, 1):
         x = bf(M_, W)
         wgu = hops.group_gate_up(bf(ff, W), bf(ff, W))
-        t = timed(lambda: hops.dense_linear(x, wgu, gated=True, act=hops.ACT_RELU))
+        t = timed_k(lambda: hops.dense_linear(x, wgu, gated=True, act=hops.ACT_RELU))
         add("hybrid", "dense_linear gated", f"M={M_} N={2 * ff} K={W}", t, 2 * ff * W * 2 + M_ * (W + ff) * 2, 2.0 * M_ * 2 * ff * W, MFMA_BF16)
         pw = quant.pack_fp16(quant.interleave_gate_up(bf(W, 2 * ff), -1))
-        t = timed(lambda: ops.linear(x, pw, None, epilogue=1))
+        t = timed_k(lambda: ops.linear(x, pw, None, epilogue=1))
         add("qwen2", "linear W16 silu_mul", f"M={M_} N={2 * ff} K={W}", t, 2 * ff * W * 2 + M_ * (W + ff) * 2, 2.0 * M_ * 2 * ff * W, MFMA_BF16)
         xo, wo = bf(M_, H * hd), bf(W, H * hd)
-        t = timed(lambda: hops.dense_linear(xo, wo, out_dtype=torch.float32))
+        t = timed_k(lambda: hops.dense_linear(xo, wo, out_dtype=torch.float32))
         add("hybrid", "dense_linear", f"M={M_} N={W} K={H * hd}", t, W * H * hd * 2 + M_ * (H * hd * 2 + W * 4), 2.0 * M_ * W * H * hd, MFMA_BF16)
         pwo = quant.pack_fp16(bf(H * hd, W))
-        t = timed(lambda: ops.linear(xo, pwo))
+        t = timed_k(lambda: ops.linear(xo, pwo))
         add("qwen2", "linear W16", f"M={M_} N={W} K={H * hd}", t, W * H * hd * 2 + M_ * (H * hd + W) * 2, 2.0 * M_ * W * H * hd, MFMA_BF16)
     # norms
     for M_ in (prompt, 8):
         x, a, b = [torch.randn(M_, W, device=dev, generator=g) for _ in range(3)]
         w1, w2 = bf(W), bf(W)
-        t = timed(lambda: hops.residual_norm(x, a, b, 0.3, w1, w2, 1e-5, weight_offset=1.0))
+        t = timed_k(lambda: hops.residual_norm(x, a, b, 0.3, w1, w2, 1e-5, weight_offset=1.0))
         add("hybrid", "residual + 2 norms (fp32 stream)", f"M={M_} W={W}", t, M_ * W * (4 * 4 + 2 * 2), 0, VALU_F32)
         xh, rh, wh = bf(M_, W).to(torch.bfloat16), bf(M_, W), bf(W)
-        t = timed(lambda: ops.add_rmsnorm(xh, rh, wh, 1e-6))
+        t = timed_k(lambda: ops.add_rmsnorm(xh, rh, wh, 1e-6))
         add("qwen2", "add + rmsnorm (16-bit stream)", f"M={M_} W={W}", t, M_ * W * 2 * 4, 0, VALU_F32)
     # attention: prefill rows over a chunk-local mask vs plain causal rows; decode at a context of `prompt`
     page, chunk = 64, 1024
@@ -193,23 +212,29 @@ def kernel_table(s, dev, prompt):
         pos = (torch.arange(T_, dtype=torch.int32, device=dev) if T_ > 1 else torch.tensor([prompt - 1], dtype=torch.int32, device=dev))
         seq = torch.zeros(T_, dtype=torch.int32, device=dev)
         q = torch.randn(T_, H * hd, device=dev, generator=g)
-        t = timed(lambda: hops.attn_rows(q, hd ** -0.5, geom, chunk, True, vf, pos, seq, bt, kc, vc, H, hd))
+        t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, chunk, True, vf, pos, seq, bt, kc, vc, H, hd))
         keys = float(sum(min(int(p) % chunk + 1, chunk) for p in pos.tolist()))
         add("hybrid", f"attn_rows {name} (chunk {chunk})", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t,
             min(prompt, chunk if T_ == 1 else prompt) * G * hd * 2 * 2 + T_ * H * hd * 6, 4.0 * keys * H * hd, MFMA_BF16)
+        if T_ > 1:
+            t0 = torch.arange(0, T_, 16, dtype=torch.int32, device=dev)
+            tn = torch.full_like(t0, 16)
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, chunk, True, vf, pos, seq, bt, t0, tn, kc, vc, H, hd))
+            add("hybrid", f"attn_tiles {name} (chunk {chunk}, MFMA)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t,
+                prompt * G * hd * 2 * 2 + T_ * H * hd * 6, 4.0 * keys * H * hd, MFMA_BF16)
         kvb = torch.randn(nblk, 2, G, page, hd, device=dev, generator=g).bfloat16()
         qh = bf(T_, H, hd)
         if T_ > 1:
             q_len = 512
             posr = torch.arange(q_len, dtype=torch.int32, device=dev) + (prompt - q_len)
             qh = bf(q_len, H, hd)
-            t = timed(lambda: ops.paged_attention_rows(qh, kvb, None, bt, posr, G, page, q_len, nblk * page))
+            t = timed_k(lambda: ops.paged_attention_rows(qh, kvb, None, bt, posr, G, page, q_len, nblk * page))
             keysq = float(sum(int(p) + 1 for p in posr.tolist()))
             add("qwen2", "paged_attn_rows prefill (last 512 rows, causal)", f"T={q_len} H={H} G={G} hd={hd} ctx={prompt}", t,
                 prompt * G * hd * 2 * 2 + q_len * H * hd * 4, 4.0 * keysq * H * hd, MFMA_BF16)
         else:
             sl = torch.tensor([prompt], dtype=torch.int32, device=dev)
-            t = timed(lambda: ops.paged_decode_attention(qh, kvb, None, bt, sl, G, page, nblk * page))
+            t = timed_k(lambda: ops.paged_decode_attention(qh, kvb, None, bt, sl, G, page, nblk * page))
             add("qwen2", "paged_decode_attn", f"B=1 H={H} G={G} hd={hd} ctx={prompt}", t, prompt * G * hd * 2 * 2, 4.0 * prompt * H * hd, MFMA_BF16)
     # recurrence: no counterpart in the Qwen2 family
     d = hd // 2
@@ -221,7 +246,7 @@ def kernel_table(s, dev, prompt):
         slot = torch.arange(nseq, dtype=torch.int32, device=dev)
         fp = torch.ones(nseq, dtype=torch.int32, device=dev)
         state = torch.zeros(nseq, H, d, hd, device=dev)
-        t = timed(lambda: hops.scan(hops.SCAN_GLA, proj, 0, H * d, 2 * H * d, z, None, None, 16.0, d ** -0.5, H, d, hd, rs, slot, fp, state, torch.bfloat16))
+        t = timed_k(lambda: hops.scan(hops.SCAN_GLA, proj, 0, H * d, 2 * H * d, z, None, None, 16.0, d ** -0.5, H, d, hd, rs, slot, fp, state, torch.bfloat16))
         add("hybrid", f"scan GLA {name}", f"T={T_} H={H} dim={d} vdim={hd}", t, T_ * (3 * H * d + 2 * H * hd) * 4 + 2 * nseq * H * d * hd * 4,
             4.0 * T_ * H * d * hd, VALU_F32)
     return rows

@@ -157,19 +157,19 @@ constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
 __device__ __forceinline__ float hy_lane_f(float v, int j) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), j)); }
 
 template <typename T>
-__global__ __launch_bounds__(256) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+__global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const T* kcache, const T* vcache, T* out) {
     constexpr int NV = HY_MAX_VDIM / 64;
     __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
-    __shared__ float m_s[4], l_s[4];
-    __shared__ float acc_s[4][HY_MAX_VDIM];
-    __shared__ float part_s[4][64][8];
+    __shared__ float m_s[16], l_s[16];
+    __shared__ float acc_s[16][HY_MAX_VDIM];
+    __shared__ float part_s[16][64][8];
     __shared__ float o_s[HY_MAX_VDIM];
-    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NW = blockDim.x >> 6, NT = blockDim.x;
     const int p = __builtin_amdgcn_readfirstlane(pos[r]), kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r] * g.max_blocks;
-    for (int d = tid; d < g.dim; d += 256) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
+    for (int d = tid; d < g.dim; d += NT) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
     __syncthreads();
     const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
     // the sink is a key of score 0 that carries no value: wave 0 starts from m = 0, l = 1
@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void hy_attn_rows_kernel(const float* q, int l
     const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 256: KPI >= 2)
     const int grp = lane / LPK, cl = (lane % LPK) * 8;
     const bool gok = grp < KPI;
-    for (int t0 = lo + wave * 64; t0 <= p; t0 += 256) {
+    for (int t0 = lo + wave * 64; t0 <= p; t0 += 64 * NW) {
         const int kj = t0 + lane;
         const bool valid = kj <= p;
         float s = -INFINITY;
@@ -271,18 +271,21 @@ __global__ __launch_bounds__(256) void hy_attn_rows_kernel(const float* q, int l
     }
     if (lane == 0) { m_s[wave] = m; l_s[wave] = l; }
     __syncthreads();
-    const float mm = fmaxf(fmaxf(m_s[0], m_s[1]), fmaxf(m_s[2], m_s[3]));
-    float w4[4], lt = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) { w4[w] = (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm); lt = __builtin_fmaf(l_s[w], w4[w], lt); }
+    float mm = m_s[0];
+    for (int w = 1; w < NW; ++w) mm = fmaxf(mm, m_s[w]);
+    float lt = 0.f;
+    for (int w = 0; w < NW; ++w) lt = __builtin_fmaf(l_s[w], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), lt);
     const float invl = lt > 0.f ? 1.f / lt : 0.f;
-    for (int c = tid; c < g.vdim; c += 256)
-        o_s[c] = (acc_s[0][c] * w4[0] + acc_s[1][c] * w4[1] + acc_s[2][c] * w4[2] + acc_s[3][c] * w4[3]) * invl;
+    for (int c = tid; c < g.vdim; c += NT) {
+        float a = 0.f;
+        for (int w = 0; w < NW; ++w) a = __builtin_fmaf(acc_s[w][c], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), a);
+        o_s[c] = a * invl;
+    }
     __syncthreads();
     T* od = out + ((size_t)r * g.H + h) * g.vdim;
     if (vfreq) {     // turn the summed values back by the query's own position
         const float fp = (float)p;
-        for (int mi = tid; mi < g.vdim / 2; mi += 256) {
+        for (int mi = tid; mi < g.vdim / 2; mi += NT) {
             int c0, c1;
             hy_pair(g.v_layout, mi, g.vdim, c0, c1);
             float sn, cs;
@@ -291,7 +294,7 @@ __global__ __launch_bounds__(256) void hy_attn_rows_kernel(const float* q, int l
             od[c0] = (T)(a * cs + b * sn); od[c1] = (T)(b * cs - a * sn);
         }
     } else {
-        for (int c = tid; c < g.vdim; c += 256) od[c] = (T)o_s[c];
+        for (int c = tid; c < g.vdim; c += NT) od[c] = (T)o_s[c];
     }
 }
 
@@ -315,32 +318,33 @@ __device__ __forceinline__ float hy_sum16(float v) {
 
 constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
 
+template <int DKM, int NCBM>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds
 __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
                                                            bf16* out) {
     __shared__ __attribute__((aligned(16))) bf16 Ph[16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Pl[16 * AT_LD];
-    __shared__ __attribute__((aligned(16))) bf16 Vt[HY_MAX_VDIM * AT_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Vt[NCBM * 16 * AT_LD];
     const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, lr = lane & 15, lq = lane >> 4;
     const int r0 = tile_row0[tile], n = tile_n[tile];
     const int p0 = pos[r0], kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r0] * g.max_blocks;
     const int DK = g.dim / 32, NCB = g.vdim / 16, VP = g.vdim / 8;
-    bf16x8 qh[8], ql[8];
+    bf16x8 qh[DKM], ql[DKM];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-        if (ks >= DK) break;
+    for (int ks = 0; ks < DKM; ++ks) {
+        if (ks >= DK) continue;
         const float* qp = q + (size_t)(r0 + min(lr, n - 1)) * ldq + h * g.dim + ks * 32 + lq * 8;
 #pragma unroll
         for (int i = 0; i < 8; ++i) { bf16 a, b; hy_split_bf16(qp[i] * scale, a, b); qh[ks][i] = a; ql[ks][i] = b; }
     }
     float m[4], l[4];
-    f32x4 o[16];
+    f32x4 o[NCBM];
 #pragma unroll
     for (int e = 0; e < 4; ++e) { m[e] = sink ? 0.f : -INFINITY; l[e] = (sink && lr == 0) ? 1.f : 0.f; }   // l: per-lane share of the row's denominator
 #pragma unroll
-    for (int cb = 0; cb < 16; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int cb = 0; cb < NCBM; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int plast = p0 + n - 1;
     const int kstart = (chunk > 0 ? (p0 / chunk) * chunk : 0) & ~31;
     for (int t0 = kstart; t0 <= plast; t0 += 32) {
@@ -349,12 +353,12 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
         for (int kb = 0; kb < 2; ++kb) {
             const int kc = min(t0 + kb * 16 + lr, plast);
             const bf16* kp = kcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.dim + lq * 8;
-            bf16x8 kf[8];
+            bf16x8 kf[DKM];
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) if (ks < DK) kf[ks] = *(const bf16x8*)(kp + ks * 32);
+            for (int ks = 0; ks < DKM; ++ks) if (ks < DK) kf[ks] = *(const bf16x8*)(kp + ks * 32);
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks)
+            for (int ks = 0; ks < DKM; ++ks)
                 if (ks < DK) {
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[ks], kf[ks], acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[ks], kf[ks], acc, 0, 0, 0);
@@ -363,7 +367,7 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
         }
         // the 32 value rows, transposed: Vt[channel][key]
         for (int i = lane; i < 32 * VP; i += 64) {
-            const int key = i / VP, c8 = (i % VP) * 8;
+            const int key = i & 31, c8 = (i >> 5) * 8;             // neighbouring lanes write neighbouring keys of one channel row
             const int kc = min(t0 + key, plast);
             const u32x4 raw = *(const u32x4*)(vcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.vdim + c8);
 #pragma unroll
@@ -393,7 +397,7 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
             l[e] = l[e] * corr + pw[0] + pw[1];
             m[e] = mn;
 #pragma unroll
-            for (int cb = 0; cb < 16; ++cb) if (cb < NCB) o[cb][e] *= corr;
+            for (int cb = 0; cb < NCBM; ++cb) if (cb < NCB) o[cb][e] *= corr;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 bf16 a, b;
@@ -404,7 +408,7 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
         __syncthreads();
         const bf16x8 ph = *(const bf16x8*)&Ph[lr * AT_LD + lq * 8], pl = *(const bf16x8*)&Pl[lr * AT_LD + lq * 8];
 #pragma unroll
-        for (int cb = 0; cb < 16; ++cb)
+        for (int cb = 0; cb < NCBM; ++cb)
             if (cb < NCB) {
                 const bf16x8 vf = *(const bf16x8*)&Vt[(cb * 16 + lr) * AT_LD + lq * 8];
                 o[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, vf, o[cb], 0, 0, 0);
@@ -420,8 +424,8 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
         const float fp = (float)(p0 + row);
         bf16* od = out + ((size_t)(r0 + row) * g.H + h) * g.vdim;
 #pragma unroll
-        for (int cb = 0; cb < 16; ++cb) {
-            if (cb >= NCB) break;
+        for (int cb = 0; cb < NCBM; ++cb) {
+            if (cb >= NCB) continue;
             const int c = cb * 16 + lr;
             float v = o[cb][e] * inv;
             if (vfreq) {          // turn back by the row's position; the partner channel sits in the next lane (interleaved) or NCB / 2 fragments away (halves)
@@ -434,7 +438,7 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
                     first = cb < half; mi = first ? c : c - g.vdim / 2;
                     float t = 0.f;
 #pragma unroll
-                    for (int k = 0; k < 16; ++k) if (k == (first ? cb + half : cb - half)) t = o[k][e] * inv;
+                    for (int k = 0; k < NCBM; ++k) if (k == (first ? cb + half : cb - half)) t = o[k][e] * inv;
                     other = t;
                 }
                 sincosf(fp * vfreq[mi], &sn, &cs);
@@ -625,7 +629,8 @@ extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, cons
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
     if (int e = hy_geom_ok(g)) return e;
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(256), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
+    const int threads = rows * g.H <= 2048 ? 1024 : 256;     // few (decode) rows: sixteen waves share a row's keys
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(threads), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
                                               pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out));
     MI355_CHECK_LAUNCH("hy_attn_rows_kernel");
     return MI355_OK;
@@ -644,8 +649,12 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
         mi355_set_error("hy_attn_tiles: bf16, dim %% 32 == 0, vdim %% 16 == 0 only (dim=%d vdim=%d dtype=%d)", g.dim, g.vdim, act_dtype);
         return MI355_ERR_UNSUPPORTED;
     }
-    hipLaunchKernelGGL(hy_attn_tiles_kernel, dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq, block_table,
-                       tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
+    if (g.dim <= 128 && g.vdim <= 128)
+        hipLaunchKernelGGL((hy_attn_tiles_kernel<4, 8>), dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
+                           block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
+    else
+        hipLaunchKernelGGL((hy_attn_tiles_kernel<8, 16>), dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
+                           block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
     MI355_CHECK_LAUNCH("hy_attn_tiles_kernel");
     return MI355_OK;
 }
