@@ -701,32 +701,6 @@ int mi355_decoder_profile(mi355_decoder_t* d, int32_t B, int32_t nsteps, float* 
  * was out of range (see mi355_rope_kv_write).  Synchronises `stream`.  0 on a healthy run; < 0 = error. */
 int64_t mi355_decoder_oob_count(mi355_decoder_t* d, mi355_stream_t stream);
 
-/* ------------------------------------------------------------------------------------------------------------------------------
- * libmi355_hybrid.so: dense linears on [out, in] weights and the kernels of the hybrid decoder family (parallel-residual layers
- * over an fp32 stream; token mixers: paged chunk-masked attention with a softmax sink and position-rotated values, and gated
- * linear recurrences with fp32 state slots).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
- * csrc/hybrid_ops.hip; the argument conventions are documented at the definitions. */
-int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
-                       int32_t out_f32, int32_t gated, int32_t act, float softcap, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_embed(const int32_t* ids, int32_t rows, const void* table, int32_t W, int32_t vocab, float* out, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_residual_norm(float* x, const float* a, const float* b, float mult, const int32_t* rows, int32_t n, int32_t W, const void* w1,
-                           const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
-                       int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
-                       void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
-                       const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
-                       const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
-                        const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0, const int32_t* tile_n,
-                        int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
-                  const void* lower, const void* fbias, float tau, float qscale, int32_t H, int32_t dim, int32_t vdim,
-                  const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,
-                  int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
-                       int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -158,7 +158,7 @@ SIGNATURES = {
     "mi355_decoder_oob_count": (C.c_int64, [vp, vp]),
 }
 
-# libmi355_hybrid.so: dense linears on [out, in] weights + the kernels of the hybrid decoder family (a library of its own, so that a
+# libmi355_hybrid.so (C-ABI: include/mi355_hybrid.h): dense linears on [out, in] weights + the kernels of the hybrid decoder family (a library of its own, so that a
 # process serving such a model builds and loads nothing else)
 HYBRID_LIB_PATH = os.path.join(_HERE, "lib", "libmi355_hybrid.so")
 ip = C.POINTER(i32)

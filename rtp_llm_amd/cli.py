@@ -27,6 +27,8 @@ def cmd_generate(a):
     import torch
     from . import registry
     eng = registry.load_engine(a.model, _dtype(a.dtype), a.device, max_tokens=a.max_tokens, max_seqs=a.max_seqs)
+    if a.graphs and hasattr(eng, "use_graphs"):
+        eng.use_graphs = True                     # decode-only steps replay a captured HIP graph
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in a.prompt_ids]
     sampling = {} if a.top_k == 1 else dict(top_k=a.top_k, top_p=a.top_p, temperature=a.temperature, seed=a.seed)
     outs = eng.generate(prompts, a.max_new_tokens, **sampling)
@@ -81,6 +83,7 @@ def main(argv=None):
     g.add_argument("--top-p", type=float, default=1.0)
     g.add_argument("--temperature", type=float, default=1.0)
     g.add_argument("--seed", type=int, default=0)
+    g.add_argument("--graphs", action="store_true", help="replay decode-only steps as captured HIP graphs (families with a ragged step function)")
     g.set_defaults(fn=cmd_generate)
     t = sub.add_parser("trace", help="replay a schedule of steps from standard input and write the logits of the asked rows")
     t.add_argument("--model", required=True)

@@ -11,6 +11,7 @@
 // Output is fp32 or the activation type.  A result row depends only on its own input row: the k order of the accumulation is fixed by
 // the kernel, never by M or by the row's place in the batch.
 #include "common.h"
+#include "../../include/mi355_hybrid.h"
 
 namespace {
 

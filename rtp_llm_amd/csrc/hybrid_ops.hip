@@ -7,6 +7,7 @@
 // sequence; a sequence carries its block-table row, its state slot and the range of its rows.  What the model states as 32-bit is fp32
 // here whatever the activation type T (bf16 or float): positions and angles, scores and softmax, norms, gates, decays, states, residual.
 #include "common.h"
+#include "../../include/mi355_hybrid.h"
 
 namespace {
 
@@ -489,31 +490,62 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
         const int d = ds * RD + j;
         s[j] = (!fresh && vok && d < p.dim) ? st[(size_t)d * p.vdim] : 0.f;
     }
+    // raw projections of the next pass are fetched into registers while the current pass is walked: element i of the staged (token, row)
+    // grid belongs to thread i % blockDim, at most RD / 4 per thread (16 tokens x DS x RD rows over 64 DS threads), value columns likewise
+    constexpr int EL = RD / 4;
+    constexpr int VE = 4;                       // value elements fetched ahead per thread; a block of fewer than four waves reads the rest late
+    float rq[EL], rk[EL], rz[EL], rv[VE];
+    auto fetch = [&](int t0) {
+        const int nt = min(TOK, r1 - t0);
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int i = tid + e * blockDim.x, t = i / dpad, d = i % dpad;
+            rq[e] = rk[e] = rz[e] = 0.f;
+            if (i < nt * dpad && d < p.dim) {
+                const float* row = p.proj + (size_t)(t0 + t) * p.ld;
+                const int hd = h * p.dim + d;
+                rq[e] = row[p.qo + hd]; rk[e] = row[p.ko + hd];
+                if (p.mode == SCAN_GLA) rz[e] = p.z[(size_t)(t0 + t) * p.ldz + hd];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+            const int i = tid + e * blockDim.x;
+            rv[e] = 0.f;
+            if (i < nt * 64 && v0 + (i & 63) < p.vdim) rv[e] = p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)];
+        }
+    };
+    if (r0 < r1) fetch(r0);
     for (int t0 = r0; t0 < r1; t0 += TOK) {
         const int nt = min(TOK, r1 - t0);
-        for (int i = tid; i < nt * dpad; i += blockDim.x) {
-            const int t = i / dpad, d = i % dpad;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+            const int i = tid + e * blockDim.x, d = i % dpad;
+            if (i >= nt * dpad) continue;
             float qv = 0.f, kv = 0.f, av = 1.f;
             if (d < p.dim) {
-                const float* row = p.proj + (size_t)(t0 + t) * p.ld;
                 const int hd = h * p.dim + d;
                 if (p.mode == SCAN_HGRN2) {
                     const float lw = (float)((const T*)p.lower)[hd];
-                    const float f = lw + (1.f - lw) * hy_sigmoid(row[p.ko + hd] + (float)((const T*)p.fbias)[hd]);
-                    qv = hy_silu(row[p.qo + hd]); av = f; kv = 1.f - f;
+                    const float f = lw + (1.f - lw) * hy_sigmoid(rk[e] + (float)((const T*)p.fbias)[hd]);
+                    qv = hy_silu(rq[e]); av = f; kv = 1.f - f;
                 } else {
-                    const float zz = p.z[(size_t)(t0 + t) * p.ldz + hd];
+                    const float zz = rz[e];
                     const float ls = fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)));       // log sigmoid(z)
-                    qv = row[p.qo + hd] * p.qscale; kv = row[p.ko + hd]; av = expf(ls / p.tau);
+                    qv = rq[e] * p.qscale; kv = rk[e]; av = expf(ls / p.tau);
                 }
             }
             q_s[i] = qv; k_s[i] = kv; a_s[i] = av;
         }
-        for (int i = tid; i < nt * 64; i += blockDim.x) {
-            const int t = i >> 6, cc = i & 63;
-            v_s[i] = (v0 + cc < p.vdim) ? p.proj[(size_t)(t0 + t) * p.ld + p.vo + h * p.vdim + v0 + cc] : 0.f;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) {
+            const int i = tid + e * blockDim.x;
+            if (i < nt * 64) v_s[i] = rv[e];
         }
+        for (int i = tid + VE * blockDim.x; i < nt * 64; i += blockDim.x)
+            v_s[i] = (v0 + (i & 63) < p.vdim) ? p.proj[(size_t)(t0 + (i >> 6)) * p.ld + p.vo + h * p.vdim + v0 + (i & 63)] : 0.f;
         __syncthreads();
+        if (t0 + TOK < r1) fetch(t0 + TOK);
         for (int t = 0; t < nt; ++t) {
             const float vt = v_s[t * 64 + c];
             const f32x4* qq = (const f32x4*)(q_s + t * dpad + ds * RD);

@@ -12,6 +12,24 @@ import hybrid_util as U  # noqa: E402
 from rtp_llm_amd.kvcache import CacheManager, PagePool  # noqa: E402
 
 
+def test_hybrid_library_builds_and_exports_every_declared_symbol():
+    import ctypes
+    import re
+    from rtp_llm_amd import _C
+    from rtp_llm_amd.build import build_hybrid
+    lib = ctypes.CDLL(build_hybrid(verbose=False))              # hipcc cross-compiles gfx950 without a GPU
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = re.sub(r"/\*.*?\*/", "", open(os.path.join(root, "include", "mi355_hybrid.h")).read(), flags=re.S)
+    declared = set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", src))
+    assert declared and declared | {"mi355_abi_version", "mi355_last_error"} == set(_C.HYBRID_SIGNATURES)
+    for name in _C.HYBRID_SIGNATURES:
+        assert hasattr(lib, name), f"{name} is not exported"
+    l = _C.hybrid_lib()
+    assert l.mi355_abi_version() == _C.ABI_VERSION
+    assert l.mi355_dense_linear(None, 0, 1, None, 8, 8, None, None, 8, 0, 0, 0, 0.0, _C.ACT_BF16, None) == _C.ERR_ARG   # argument errors need no GPU
+    assert b"dense_linear" in l.mi355_last_error()
+
+
 def test_page_pool_reuses_what_came_back():
     p = PagePool(4)
     assert p.take(3) == [0, 1, 2]
