@@ -300,7 +300,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
 }
 
 // ------------------------------------------------------------------------------------------------ attention for prompt portions: MFMA tiles (bf16 cache)
-// One wave per (tile of up to 16 consecutive rows of one sequence, head).  Keys go by 32: S = Q K^T with v_mfma_f32_16x16x32_bf16 (K fragments
+// One wave per (tile of up to 16 consecutive rows of one sequence, head); up to four heads of one key/value head form a block.  Keys go by 32: S = Q K^T with v_mfma_f32_16x16x32_bf16 (K fragments
 // straight from the cache: 8 consecutive channels per lane), mask and online softmax on the fp32 accumulator fragments, then O += P V with P
 // passed through LDS into the A layout and the 32 value rows transposed through LDS into the B layout.  Scores and weights stay 32-bit: the
 // fp32 queries (scaled) and the fp32 weights enter the matrix unit as an exact sum of two bf16 terms (high part + remainder), the cached
@@ -320,14 +320,18 @@ __device__ __forceinline__ float hy_sum16(float v) {
 constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
 
 template <int DKM, int NCBM>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds
-__global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+__global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
                                                            bf16* out) {
-    __shared__ __attribute__((aligned(16))) bf16 Ph[16 * AT_LD];
-    __shared__ __attribute__((aligned(16))) bf16 Pl[16 * AT_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Ph_all[4][16 * AT_LD];
+    __shared__ __attribute__((aligned(16))) bf16 Pl_all[4][16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Vt[NCBM * 16 * AT_LD];
-    const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, lr = lane & 15, lq = lane >> 4;
+    // the waves of a block are query heads that share one key/value head: they walk the same keys and share the transposed value tile
+    const int wave = threadIdx.x >> 6, NWV = blockDim.x >> 6;
+    const int tile = blockIdx.x, h = blockIdx.y * NWV + wave, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
+    bf16* Ph = Ph_all[wave];
+    bf16* Pl = Pl_all[wave];
     const int r0 = tile_row0[tile], n = tile_n[tile];
     const int p0 = pos[r0], kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r0] * g.max_blocks;
@@ -367,7 +371,7 @@ __global__ __launch_bounds__(64) void hy_attn_tiles_kernel(const float* q, int l
             s[kb] = acc;
         }
         // the 32 value rows, transposed: Vt[channel][key]
-        for (int i = lane; i < 32 * VP; i += 64) {
+        for (int i = threadIdx.x; i < 32 * VP; i += blockDim.x) {
             const int key = i & 31, c8 = (i >> 5) * 8;             // neighbouring lanes write neighbouring keys of one channel row
             const int kc = min(t0 + key, plast);
             const u32x4 raw = *(const u32x4*)(vcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.vdim + c8);
@@ -681,11 +685,12 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
         mi355_set_error("hy_attn_tiles: bf16, dim %% 32 == 0, vdim %% 16 == 0 only (dim=%d vdim=%d dtype=%d)", g.dim, g.vdim, act_dtype);
         return MI355_ERR_UNSUPPORTED;
     }
+    const int gq = g.H / g.G, nwv = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;       // query heads of one key/value head per block
     if (g.dim <= 128 && g.vdim <= 128)
-        hipLaunchKernelGGL((hy_attn_tiles_kernel<4, 8>), dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
+        hipLaunchKernelGGL((hy_attn_tiles_kernel<4, 8>), dim3(tiles, g.H / nwv), dim3(64 * nwv), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
                            block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
     else
-        hipLaunchKernelGGL((hy_attn_tiles_kernel<8, 16>), dim3(tiles, g.H), dim3(64), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
+        hipLaunchKernelGGL((hy_attn_tiles_kernel<8, 16>), dim3(tiles, g.H / nwv), dim3(64 * nwv), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
                            block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
     MI355_CHECK_LAUNCH("hy_attn_tiles_kernel");
     return MI355_OK;
