@@ -319,7 +319,7 @@ __device__ __forceinline__ float hy_sum16(float v) {
 
 constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
 
-template <int DKM, int NCBM>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds
+template <int DKM, int NCBM, int NWV>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds; waves per block
 __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
@@ -328,7 +328,8 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     __shared__ __attribute__((aligned(16))) bf16 Pl_all[4][16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Vt[NCBM * 16 * AT_LD];
     // the waves of a block are query heads that share one key/value head: they walk the same keys and share the transposed value tile
-    const int wave = threadIdx.x >> 6, NWV = blockDim.x >> 6;
+    const int wave = threadIdx.x >> 6;
+    constexpr int VEM = NCBM / NWV;                           // 32 VP pieces of 16 bytes over 64 NWV threads: at most NCBM / NWV per thread
     const int tile = blockIdx.x, h = blockIdx.y * NWV + wave, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
     bf16* Ph = Ph_all[wave];
     bf16* Pl = Pl_all[wave];
@@ -336,6 +337,11 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     const int p0 = pos[r0], kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r0] * g.max_blocks;
     const int DK = g.dim / 32, NCB = g.vdim / 16, VP = g.vdim / 8;
+    const int psh = (g.page & (g.page - 1)) == 0 ? __builtin_ctz(g.page) : -1;       // page size a power of two: shifts instead of divisions
+    auto cache_row = [&](int kc) {
+        const int pi = psh >= 0 ? kc >> psh : kc / g.page, po = psh >= 0 ? kc & (g.page - 1) : kc % g.page;
+        return (size_t)(bt[pi] * g.G + kvh) * g.page + po;
+    };
     bf16x8 qh[DKM], ql[DKM];
 #pragma unroll
     for (int ks = 0; ks < DKM; ++ks) {
@@ -351,41 +357,63 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 #pragma unroll
     for (int cb = 0; cb < NCBM; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int plast = p0 + n - 1;
+    int rlo4[4];                                              // first visible position of the lane's four rows
+#pragma unroll
+    for (int e = 0; e < 4; ++e) rlo4[e] = chunk > 0 ? ((p0 + lq * 4 + e) / chunk) * chunk : 0;
     const int kstart = (chunk > 0 ? (p0 / chunk) * chunk : 0) & ~31;
+    // the key fragments and raw value rows of the next 32 keys are fetched while the current 32 are worked on
+    bf16x8 kn[2][DKM];
+    u32x4 vn[VEM];
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int kc = min(t0 + kb * 16 + lr, plast);
+            const bf16* kp = kcache + cache_row(kc) * g.dim + lq * 8;
+#pragma unroll
+            for (int ks = 0; ks < DKM; ++ks) if (ks < DK) kn[kb][ks] = *(const bf16x8*)(kp + ks * 32);
+        }
+#pragma unroll
+        for (int e = 0; e < VEM; ++e) {
+            const int i = threadIdx.x + e * 64 * NWV;
+            if (i < 32 * VP) {
+                const int kc = min(t0 + (i & 31), plast);
+                vn[e] = *(const u32x4*)(vcache + cache_row(kc) * g.vdim + (i >> 5) * 8);
+            }
+        }
+    };
+    fetch(kstart);
     for (int t0 = kstart; t0 <= plast; t0 += 32) {
         f32x4 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            const int kc = min(t0 + kb * 16 + lr, plast);
-            const bf16* kp = kcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.dim + lq * 8;
-            bf16x8 kf[DKM];
-#pragma unroll
-            for (int ks = 0; ks < DKM; ++ks) if (ks < DK) kf[ks] = *(const bf16x8*)(kp + ks * 32);
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < DKM; ++ks)
                 if (ks < DK) {
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[ks], kf[ks], acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[ks], kf[ks], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[ks], kn[kb][ks], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[ks], kn[kb][ks], acc, 0, 0, 0);
                 }
             s[kb] = acc;
         }
-        // the 32 value rows, transposed: Vt[channel][key]
-        for (int i = threadIdx.x; i < 32 * VP; i += blockDim.x) {
-            const int key = i & 31, c8 = (i >> 5) * 8;             // neighbouring lanes write neighbouring keys of one channel row
-            const int kc = min(t0 + key, plast);
-            const u32x4 raw = *(const u32x4*)(vcache + ((size_t)(bt[kc / g.page] * g.G + kvh) * g.page + kc % g.page) * g.vdim + c8);
+        // the 32 value rows, transposed: Vt[channel][key]; neighbouring lanes write neighbouring keys of one channel row
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *(uint16_t*)&Vt[(c8 + 2 * j) * AT_LD + key] = (uint16_t)(raw[j] & 0xFFFFu);
-                *(uint16_t*)&Vt[(c8 + 2 * j + 1) * AT_LD + key] = (uint16_t)(raw[j] >> 16);
+        for (int e = 0; e < VEM; ++e) {
+            const int i = threadIdx.x + e * 64 * NWV;
+            if (i < 32 * VP) {
+                const int key = i & 31, c8 = (i >> 5) * 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    *(uint16_t*)&Vt[(c8 + 2 * j) * AT_LD + key] = (uint16_t)(vn[e][j] & 0xFFFFu);
+                    *(uint16_t*)&Vt[(c8 + 2 * j + 1) * AT_LD + key] = (uint16_t)(vn[e][j] >> 16);
+                }
             }
         }
+        if (t0 + 32 <= plast) fetch(t0 + 32);                  // in flight during the softmax and the second product
         // mask, running maximum, weights; fragment element e is row 4 lq + e, the lane's key columns are kb * 16 + lr
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = lq * 4 + e, rpos = p0 + row;
-            const int rlo = chunk > 0 ? (rpos / chunk) * chunk : 0;
+            const int rlo = rlo4[e];
             float sv[2];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
@@ -686,12 +714,12 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
         return MI355_ERR_UNSUPPORTED;
     }
     const int gq = g.H / g.G, nwv = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;       // query heads of one key/value head per block
-    if (g.dim <= 128 && g.vdim <= 128)
-        hipLaunchKernelGGL((hy_attn_tiles_kernel<4, 8>), dim3(tiles, g.H / nwv), dim3(64 * nwv), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
-                           block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
-    else
-        hipLaunchKernelGGL((hy_attn_tiles_kernel<8, 16>), dim3(tiles, g.H / nwv), dim3(64 * nwv), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq, pos, seq,
-                           block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out);
+#define HY_TILES(DKM_, NCBM_, NWV_)                                                                                                            \
+    hipLaunchKernelGGL((hy_attn_tiles_kernel<DKM_, NCBM_, NWV_>), dim3(tiles, g.H / NWV_), dim3(64 * NWV_), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, \
+                       sink, vfreq, pos, seq, block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out)
+    if (g.dim <= 128 && g.vdim <= 128) { if (nwv == 4) HY_TILES(4, 8, 4); else if (nwv == 2) HY_TILES(4, 8, 2); else HY_TILES(4, 8, 1); }
+    else                               { if (nwv == 4) HY_TILES(8, 16, 4); else if (nwv == 2) HY_TILES(8, 16, 2); else HY_TILES(8, 16, 1); }
+#undef HY_TILES
     MI355_CHECK_LAUNCH("hy_attn_tiles_kernel");
     return MI355_OK;
 }
