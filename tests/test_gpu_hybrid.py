@@ -99,6 +99,9 @@ ALONE = {
     "gla": U.gla_layer(ff=None),
     "gla_tau_one_rank_four": U.gla_layer(heads=3, dim=40, vdim=24, tau=1.0, ff=None, rank=4),
     "mlp_unaligned_channels": U.hgrn2_layer(heads=1, dim=8, vdim=8, ff=40),
+    "gla_key_size_160": U.gla_layer(heads=2, dim=160, vdim=16, ff=None),
+    "hgrn2_key_size_320": U.hgrn2_layer(heads=1, dim=320, vdim=72, ff=None),
+    "attention_key_size_264": U.attention_layer(heads=2, kv_heads=1, dim=264, vdim=8, rot_dims=64, chunk=30, ff=None),
 }
 
 
