@@ -306,15 +306,21 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
 // fp32 queries (scaled) and the fp32 weights enter the matrix unit as an exact sum of two bf16 terms (high part + remainder), the cached
 // keys and values are bf16 as stored, every accumulation is fp32.
 __device__ __forceinline__ void hy_split_bf16(float x, bf16& hi, bf16& lo) { hi = (bf16)x; lo = (bf16)(x - (float)hi); }
+// reductions over the 16 lanes of a DPP row (the lanes that hold one fragment row): quad swaps, then the half-row and row mirrors
+template <int CTRL> __device__ __forceinline__ float hy_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float hy_max16(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, hy_dpp<0xB1>(v));      // quad_perm [1,0,3,2]
+    v = fmaxf(v, hy_dpp<0x4E>(v));      // quad_perm [2,3,0,1]
+    v = fmaxf(v, hy_dpp<0x141>(v));     // row_half_mirror
+    return fmaxf(v, hy_dpp<0x140>(v));  // row_mirror
 }
 __device__ __forceinline__ float hy_sum16(float v) {
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += hy_dpp<0xB1>(v);
+    v += hy_dpp<0x4E>(v);
+    v += hy_dpp<0x141>(v);
+    return v + hy_dpp<0x140>(v);
 }
 
 constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
