@@ -348,13 +348,15 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
         const int pi = psh >= 0 ? kc >> psh : kc / g.page, po = psh >= 0 ? kc & (g.page - 1) : kc % g.page;
         return (size_t)(bt[pi] * g.G + kvh) * g.page + po;
     };
+    // scores are kept times log2(e): the weights are then 2^(s - m), one v_exp_f32 each; the sink (score 0) and the ratios are unchanged
+    const float scale2 = scale * 1.44269504088896340736f;
     bf16x8 qh[DKM], ql[DKM];
 #pragma unroll
     for (int ks = 0; ks < DKM; ++ks) {
         if (ks >= DK) continue;
         const float* qp = q + (size_t)(r0 + min(lr, n - 1)) * ldq + h * g.dim + ks * 32 + lq * 8;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { bf16 a, b; hy_split_bf16(qp[i] * scale, a, b); qh[ks][i] = a; ql[ks][i] = b; }
+        for (int i = 0; i < 8; ++i) { bf16 a, b; hy_split_bf16(qp[i] * scale2, a, b); qh[ks][i] = a; ql[ks][i] = b; }
     }
     float m[4], l[4];
     f32x4 o[NCBM];
@@ -363,6 +365,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 #pragma unroll
     for (int cb = 0; cb < NCBM; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int plast = p0 + n - 1;
+    const int rlo_last = chunk > 0 ? (plast / chunk) * chunk : 0;
     int rlo4[4];                                              // first visible position of the lane's four rows
 #pragma unroll
     for (int e = 0; e < 4; ++e) rlo4[e] = chunk > 0 ? ((p0 + lq * 4 + e) / chunk) * chunk : 0;
@@ -415,6 +418,8 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
             }
         }
         if (t0 + 32 <= plast) fetch(t0 + 32);                  // in flight during the softmax and the second product
+        // a step whose 32 keys are visible to every row of the tile (behind the first row, inside the last row's block) needs no mask
+        const bool interior = t0 + 31 <= p0 && t0 >= rlo_last;
         // mask, running maximum, weights; fragment element e is row 4 lq + e, the lane's key columns are kb * 16 + lr
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -424,14 +429,14 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 const int kpos = t0 + kb * 16 + lr;
-                sv[kb] = (row < n && kpos <= rpos && kpos >= rlo) ? s[kb][e] : -INFINITY;
+                sv[kb] = (interior || (row < n && kpos <= rpos && kpos >= rlo)) ? s[kb][e] : -INFINITY;
             }
             const float mn = fmaxf(m[e], hy_max16(fmaxf(sv[0], sv[1])));
             float pw[2] = {0.f, 0.f}, corr = 1.f;
             if (mn != -INFINITY) {
-                corr = (m[e] == -INFINITY) ? 0.f : expf(m[e] - mn);
+                corr = (m[e] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m[e] - mn);
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) pw[kb] = (sv[kb] == -INFINITY) ? 0.f : expf(sv[kb] - mn);
+                for (int kb = 0; kb < 2; ++kb) pw[kb] = (sv[kb] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sv[kb] - mn);
             }
             l[e] = l[e] * corr + pw[0] + pw[1];
             m[e] = mn;
