@@ -47,33 +47,59 @@ __global__ __launch_bounds__(256) void hy_embed_kernel(const int32_t* ids, const
 }
 
 // ------------------------------------------------------------------------------------------------ residual update + one or two norms
+template <typename T> __device__ __forceinline__ void hy_load4(const T* p, float (&o)[4]);
+template <> __device__ __forceinline__ void hy_load4<float>(const float* p, float (&o)[4]) { const f32x4 v = *(const f32x4*)p; o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3]; }
+template <> __device__ __forceinline__ void hy_load4<bf16>(const bf16* p, float (&o)[4]) {
+    const u32x2 v = *(const u32x2*)p;
+    o[0] = act_lo<true>(v[0]); o[1] = act_hi<true>(v[0]); o[2] = act_lo<true>(v[1]); o[3] = act_hi<true>(v[1]);
+}
+template <typename T> __device__ __forceinline__ void hy_store4(T* p, const float (&o)[4]);
+template <> __device__ __forceinline__ void hy_store4<float>(float* p, const float (&o)[4]) { *(f32x4*)p = f32x4{o[0], o[1], o[2], o[3]}; }
+template <> __device__ __forceinline__ void hy_store4<bf16>(bf16* p, const float (&o)[4]) { *(u32x2*)p = u32x2{act_pack<true>(o[0], o[1]), act_pack<true>(o[2], o[3])}; }
+
 // x[src] <- x[src] + mult * (a[src] + b[src]) (written back unless rows are gathered), then h1 = norm(x) * (off + w1), h2 likewise.
-template <typename T>
+// VEC: W % 4 == 0, four channels per thread and trip (16-byte accesses on the fp32 stream).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, float mult, const int32_t* rows,
                                                                const T* w1, const T* w2, float off, float eps, int W, T* h1, T* h2) {
-    extern __shared__ float hy_xs[];
+    extern __shared__ __attribute__((aligned(16))) float hy_xs[];
     __shared__ float red[4];
     const int r = blockIdx.x, src = rows ? rows[r] : r;
+    constexpr int V = VEC ? 4 : 1;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < W; c += 256) {
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
         const size_t i = (size_t)src * W + c;
-        float v = x[i];
+        float v[4], ya[4] = {0.f, 0.f, 0.f, 0.f}, yb[4] = {0.f, 0.f, 0.f, 0.f};
+        if (VEC) { hy_load4<float>(x + i, v); if (a) hy_load4<float>(a + i, ya); if (b) hy_load4<float>(b + i, yb); }
+        else     { v[0] = x[i]; if (a) ya[0] = a[i]; if (b) yb[0] = b[i]; }
         if (a || b) {
-            const float y = (a ? a[i] : 0.f) + (b ? b[i] : 0.f);
-            v = v + mult * y;
-            if (!rows) x[i] = v;
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[e] = v[e] + mult * (ya[e] + yb[e]);
+            if (!rows) { if (VEC) hy_store4<float>(x + i, v); else x[i] = v[0]; }
         }
-        hy_xs[c] = v;
-        ss = __builtin_fmaf(v, v, ss);
+#pragma unroll
+        for (int e = 0; e < V; ++e) { hy_xs[c + e] = v[e]; ss = __builtin_fmaf(v[e], v[e], ss); }
     }
     ss = hy_wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float inv = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)W + eps);
-    for (int c = threadIdx.x; c < W; c += 256) {
-        const float u = hy_xs[c] * inv;
-        if (h1) h1[(size_t)r * W + c] = (T)(u * (off + (float)w1[c]));
-        if (h2) h2[(size_t)r * W + c] = (T)(u * (off + (float)w2[c]));
+    for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+        float u[4], g1[4], g2[4], o1[4], o2[4];
+#pragma unroll
+        for (int e = 0; e < V; ++e) u[e] = hy_xs[c + e] * inv;
+        if (h1) {
+            if (VEC) hy_load4<T>(w1 + c, g1); else g1[0] = (float)w1[c];
+#pragma unroll
+            for (int e = 0; e < V; ++e) o1[e] = u[e] * (off + g1[e]);
+            if (VEC) hy_store4<T>(h1 + (size_t)r * W + c, o1); else h1[(size_t)r * W + c] = (T)o1[0];
+        }
+        if (h2) {
+            if (VEC) hy_load4<T>(w2 + c, g2); else g2[0] = (float)w2[c];
+#pragma unroll
+            for (int e = 0; e < V; ++e) o2[e] = u[e] * (off + g2[e]);
+            if (VEC) hy_store4<T>(h2 + (size_t)r * W + c, o2); else h2[(size_t)r * W + c] = (T)o2[0];
+        }
     }
 }
 
@@ -674,8 +700,13 @@ extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, 
                                       mi355_stream_t stream) {
     MI355_CHECK_ARG(x && n > 0 && W > 0 && (!h1 || w1) && (!h2 || w2), "hy_residual_norm: n=%d W=%d", n, W);
     MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_residual_norm: W=%d too wide for one block", W);
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_residual_norm_kernel<T>, dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
-                                              (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
+    auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
+    if (W % 4 == 0 && al(x) && al(a) && al(b) && al(w1) && al(w2) && al(h1) && al(h2))
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
+                                                  (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
+    else
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
+                                                  (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
     MI355_CHECK_LAUNCH("hy_residual_norm_kernel");
     return MI355_OK;
 }

@@ -66,6 +66,7 @@ class StepBatch:
     want: torch.Tensor                   # rows whose logits are computed
     tile_row0: Optional[torch.Tensor] = None   # tiles of at most 16 consecutive rows of one sequence covering every row: first row ...
     tile_n: Optional[torch.Tensor] = None      # ... and row count (the matrix-core attention for prompt portions works on them)
+    host: Optional[torch.Tensor] = None        # the pinned buffer all index fields were uploaded from (one copy per step)
 
 
 def rotary_steps(n_pairs: int, span: int, base: float, device) -> torch.Tensor:

@@ -84,16 +84,35 @@ class ServingEngine:
                 want.append(base + int(w))
             tables.append(sc.pages)
         width = max(8, -(-max(len(t) for t in tables) // 8) * 8)
-        bt = torch.zeros(len(tables), width, dtype=torch.int32)
-        for i, t in enumerate(tables):
-            bt[i, : len(t)] = torch.tensor(t, dtype=torch.int32)
-        i32 = lambda v: torch.tensor(v, dtype=torch.int32).to(self.device, non_blocking=True)
         t0, tn = [], []
         for a, b in zip(row_start[:-1], row_start[1:]):           # tiles of at most 16 consecutive rows of one sequence
             t0 += list(range(a, b, 16))
             tn += [min(16, b - r) for r in range(a, b, 16)]
-        return StepBatch(i32(tokens), i32(pos), i32(seq), i32(row_start), i32(slot), i32(first), bt.to(self.device, non_blocking=True), i32(want),
-                         i32(t0), i32(tn))
+        bt = []
+        for t in tables:
+            bt += t + [0] * (width - len(t))
+        # every index array of the step travels in ONE pinned int32 buffer and one copy; the fields are views into the device copy
+        parts = [tokens, pos, seq, row_start, slot, first, bt, want, t0, tn]
+        offs = [0]
+        for part in parts:
+            offs.append(offs[-1] + (len(part) + 3) // 4 * 4)      # 16-byte aligned fields
+        host = torch.zeros(offs[-1], dtype=torch.int32, pin_memory=self.device.type == "cuda")
+        for o, part in zip(offs, parts):
+            if part:
+                host[o:o + len(part)] = torch.tensor(part, dtype=torch.int32)
+        batch = self.batch_views(host.to(self.device, non_blocking=True), [len(part) for part in parts], len(tables), width)
+        batch.host = host
+        return batch
+
+    @staticmethod
+    def batch_views(buf: torch.Tensor, sizes, nseq: int, width: int) -> StepBatch:
+        """The StepBatch whose fields are views of `buf` (layout of _build: fields in StepBatch order, each padded to 4 elements)."""
+        views, o = [], 0
+        for n in sizes:
+            views.append(buf[o:o + n])
+            o += (n + 3) // 4 * 4
+        views[6] = views[6].view(nseq, width)
+        return StepBatch(*views)
 
     def run_step(self, entries, collect: Optional[list] = None) -> Optional[torch.Tensor]:
         """Run the entries as one batch; -> fp32 logits [wanted rows, vocab] in the order of the entries and their wants (None if none)."""
@@ -112,19 +131,20 @@ class ServingEngine:
     def _replay_decode(self, batch: StepBatch) -> torch.Tensor:
         """The decode step as a graph: captured once per shape over static input tensors (capture runs nothing, so the recurrent states
         move only on replay), then fed by copies into those tensors."""
-        fields = ("tokens", "pos", "seq", "row_start", "slot", "first_pos", "block_table", "want", "tile_row0", "tile_n")
         key = (batch.slot.numel(), batch.block_table.shape[1])
         ent = self._graphs.get(key)
         if ent is None:
-            static = StepBatch(*[getattr(batch, f).clone() for f in fields])
+            buf = torch.empty_like(batch.host, device=self.device)
+            buf.copy_(batch.host)
+            nseq, width = key
+            static = self.batch_views(buf, [nseq, nseq, nseq, nseq + 1, nseq, nseq, nseq * width, nseq, nseq, nseq], nseq, width)
             torch.cuda.synchronize()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 out = self.model.forward(static, self.tensors)
-            ent = self._graphs[key] = (g, static, out)
-        g, static, out = ent
-        for f in fields:
-            getattr(static, f).copy_(getattr(batch, f), non_blocking=True)
+            ent = self._graphs[key] = (g, buf, out)
+        g, buf, out = ent
+        buf.copy_(batch.host, non_blocking=True)              # one copy feeds every index array of the captured step
         g.replay()
         return out.clone()
 
