@@ -1,7 +1,7 @@
 """Command line of the package.
 
     python -m rtp_llm_amd.cli generate --model DIR --prompt-ids 5,17,3 [--prompt-ids ...] --max-new-tokens N [--dtype bfloat16|float32]
-                                       [--top-k K --top-p P --temperature T --seed S]
+                                       [--top-k K --top-p P --temperature T --seed S] [--no-graphs]
     python -m rtp_llm_amd.cli trace --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N      (steps on standard input)
     python -m rtp_llm_amd.cli families
 
@@ -27,7 +27,7 @@ def cmd_generate(a):
     import torch
     from . import registry
     eng = registry.load_engine(a.model, _dtype(a.dtype), a.device, max_tokens=a.max_tokens, max_seqs=a.max_seqs)
-    if a.graphs and hasattr(eng, "use_graphs"):
+    if not a.no_graphs and hasattr(eng, "use_graphs"):
         eng.use_graphs = True                     # decode-only steps replay a captured HIP graph
     prompts = [[int(t) for t in p.split(",") if t.strip()] for p in a.prompt_ids]
     sampling = {} if a.top_k == 1 else dict(top_k=a.top_k, top_p=a.top_p, temperature=a.temperature, seed=a.seed)
@@ -83,7 +83,7 @@ def main(argv=None):
     g.add_argument("--top-p", type=float, default=1.0)
     g.add_argument("--temperature", type=float, default=1.0)
     g.add_argument("--seed", type=int, default=0)
-    g.add_argument("--graphs", action="store_true", help="replay decode-only steps as captured HIP graphs (families with a ragged step function)")
+    g.add_argument("--no-graphs", action="store_true", help="run decode-only steps eagerly instead of replaying captured HIP graphs (families with a ragged step function)")
     g.set_defaults(fn=cmd_generate)
     t = sub.add_parser("trace", help="replay a schedule of steps from standard input and write the logits of the asked rows")
     t.add_argument("--model", required=True)
