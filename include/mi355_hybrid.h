@@ -14,7 +14,8 @@ extern "C" {
 /* ------------------------------------------------------------------------------------------------------------------------------
  * libmi355_hybrid.so: dense linears on [out, in] weights and the kernels of the hybrid decoder family (parallel-residual layers
  * over an fp32 stream; token mixers: paged chunk-masked attention with a softmax sink and position-rotated values, and gated
- * linear recurrences with fp32 state slots).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
+ * linear recurrences with fp32 state slots; low-rank latent attention over one cached row per token, fixed-decay retention, PolyNorm,
+ * sigmoid-gated branches, group-limited mixtures of experts over grouped linears).  act_dtype is MI355_ACT_BF16 or MI355_ACT_F32.  Sources: csrc/gemm_dense.hip,
  * csrc/hybrid_ops.hip; the argument conventions are documented at the definitions. */
 int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
                        int32_t out_f32, int32_t gated, int32_t act, float softcap, int32_t act_dtype, mi355_stream_t stream);
@@ -24,10 +25,10 @@ int mi355_hy_residual_norm(float* x, const float* a, const float* b, float mult,
 int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const int32_t* geom, const float* kfreq, const float* vfreq,
                        int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
                        void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                        const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
                        const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                         const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0, const int32_t* tile_n,
                         int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
@@ -36,6 +37,26 @@ int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32
                   int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
                        int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream);
+int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
+                        int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs, int64_t ys, const int32_t* offs,
+                        const int32_t* gather, mi355_stream_t stream);
+int mi355_hy_gated_residual_norm(float* x, const float* a, const float* b, const float* gate, int32_t ldg, float mult, const int32_t* rows, int32_t n,
+                                 int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
+                                 mi355_stream_t stream);
+int mi355_hy_latent_prep(const float* proj, int32_t ld, int32_t doff, const int32_t* geom, const float* freq, float mag, const void* cw, float eps,
+                         const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, void* qn, float* qabs, void* cache,
+                         int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_rotary(float* buf, int32_t ld, int32_t rows, int32_t off0, int32_t heads0, int32_t dim0, float scale0, int32_t off1, int32_t heads1,
+                    int32_t dim1, float scale1, int32_t rdims, int32_t layout, const float* freq, float mag, const int32_t* pos, mi355_stream_t stream);
+int mi355_hy_polynorm(const float* z, int32_t ld, int32_t rows, int32_t n, float ca, float cb, float cc, float ce, float eps, void* out, int32_t ldo,
+                      int32_t act_dtype, mi355_stream_t stream);
+int mi355_hy_gate_mul(const float* o, int32_t rows, int32_t n, const float* gate, int32_t ldg, int32_t goff, void* out, int32_t act_dtype,
+                      mi355_stream_t stream);
+int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                       mi355_stream_t stream);
+int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, int32_t E, int32_t* offs, int32_t* src_row, int32_t* place_of, mi355_stream_t stream);
+int mi355_hy_moe_combine(const float* y, int32_t tokens, int32_t W, const int32_t* place_of, const float* wts, int32_t top, const float* extra, float* out,
+                         mi355_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -25,7 +25,23 @@ struct DenseParams {
     int out_f32;
     float softcap;   // > 0: y = cap * tanh(y / cap)
     int vec;         // 16-byte loads allowed (alignment and K % 8 == 0 checked on the host)
+    // groups (tile kernels, blockIdx.z): group g multiplies its rows by the weight w + g * ws (bias + g * N) and writes columns ys * g + ...
+    // of y; it reads x from column xs * g on.  Its rows are all M rows, or rows offs[g] .. offs[g + 1] - 1 of a list sorted by group, whose
+    // entry r reads x row gather[r] (identity without gather) and writes y row r.
+    int G;
+    long long xs, ws, ys;
+    const int32_t* offs; const int32_t* gather;
 };
+
+// rows [rbeg, rend) of the block's group and its operand bases
+struct DnGroup { int rbeg, rend; long long xo, wo, yo; int bo; };
+__device__ __forceinline__ DnGroup dn_group(const DenseParams& p) {
+    const int g = blockIdx.z;
+    DnGroup r;
+    r.rbeg = p.offs ? p.offs[g] : 0; r.rend = p.offs ? p.offs[g + 1] : p.M;
+    r.xo = p.xs * g; r.wo = p.ws * g; r.yo = p.ys * g; r.bo = g * p.N;
+    return r;
+}
 
 __device__ __forceinline__ float dn_act(float g, int act) {
     if (act == DN_ACT_RELU) return g > 0.f ? g : 0.f;
@@ -47,7 +63,7 @@ constexpr int TB_M = 64, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;   // LDS row s
 
 __device__ __forceinline__ u32x4 dn_chunk_bf16(const bf16* base, int row, int rows, int k, int K, int ld, int vec) {
     u32x4 z = {0u, 0u, 0u, 0u};
-    if (row >= rows || k >= K) return z;
+    if (row >= rows || k >= K) return z;     // row 0x7fffffff: no row
     const bf16* p = base + (size_t)row * ld + k;
     if (vec) return *(const u32x4*)p;
     uint16_t e[8];
@@ -64,9 +80,18 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
     __shared__ __attribute__((aligned(16))) bf16 Bs[TB_N * TB_LD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = wave >> 1;                       // wave tile: rows wm*32.., cols wn*64..
-    const int m0 = blockIdx.y * TB_M, n0 = blockIdx.x * TB_N;
-    const bf16* X = (const bf16*)p.x;
-    const bf16* W = (const bf16*)p.w;
+    const DnGroup gr = dn_group(p);
+    const int m0 = gr.rbeg + blockIdx.y * TB_M, n0 = blockIdx.x * TB_N;
+    if (m0 >= gr.rend) return;
+    const bf16* X = (const bf16*)p.x + gr.xo;
+    const bf16* W = (const bf16*)p.w + gr.wo;
+    const bf16* Bi = p.bias ? (const bf16*)p.bias + gr.bo : nullptr;
+    int arow[2];                                                   // x rows this thread stages (past the group's end: none)
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = m0 + ((tid + i * 256) >> 3);
+        arow[i] = r < gr.rend ? (p.gather ? p.gather[r] : r) : 0x7fffffff;
+    }
     f32x4 acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -76,7 +101,7 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
     u32x4 ra[2], rb[4];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) { const int c = tid + i * 256; ra[i] = dn_chunk_bf16(X, m0 + (c >> 3), p.M, k0 + (c & 7) * 8, p.K, p.ldx, p.vec); }
+        for (int i = 0; i < 2; ++i) { const int c = tid + i * 256; ra[i] = dn_chunk_bf16(X, arow[i], 0x7fffffff, k0 + (c & 7) * 8, p.K, p.ldx, p.vec); }
 #pragma unroll
         for (int i = 0; i < 4; ++i) { const int c = tid + i * 256; rb[i] = dn_chunk_bf16(W, n0 + (c >> 3), p.N, k0 + (c & 7) * 8, p.K, p.K, p.vec); }
     };
@@ -110,15 +135,15 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = m0 + wm * 32 + i * 16 + rq + e;
-            if (row >= p.M) continue;
+            if (row >= gr.rend) continue;
             if (p.gated) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int ng = n0 + wn * 64 + j * 16 + cl;         // weight row of the gate; its up row is ng + 32
                     if (ng + 32 >= p.N) continue;
                     float g = acc[i][j][e], u = acc[i][j + 2][e];
-                    if (p.bias) { g += dn_ld((const bf16*)p.bias + ng); u += dn_ld((const bf16*)p.bias + ng + 32); }
-                    dn_store<bf16>(p, row, (ng >> 6) * 32 + (ng & 31), dn_act(g, p.act) * u);
+                    if (Bi) { g += dn_ld(Bi + ng); u += dn_ld(Bi + ng + 32); }
+                    dn_store<bf16>(p, row, (int)gr.yo + (ng >> 6) * 32 + (ng & 31), dn_act(g, p.act) * u);
                 }
             } else {
 #pragma unroll
@@ -126,8 +151,8 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
                     const int n = n0 + wn * 64 + j * 16 + cl;
                     if (n >= p.N) continue;
                     float v = acc[i][j][e];
-                    if (p.bias) v += dn_ld((const bf16*)p.bias + n);
-                    dn_store<bf16>(p, row, n, dn_act(v, p.act));
+                    if (Bi) v += dn_ld(Bi + n);
+                    dn_store<bf16>(p, row, (int)gr.yo + n, dn_act(v, p.act));
                 }
             }
         }
@@ -150,16 +175,20 @@ __global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
     __shared__ __attribute__((aligned(16))) float As[TF_K * TF_LD];   // [k][m]
     __shared__ __attribute__((aligned(16))) float Bs[TF_K * TF_LD];   // [k][n]
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
-    const int m0 = blockIdx.y * TF_M, n0 = blockIdx.x * TF_N;
-    const float* X = (const float*)p.x;
-    const float* W = (const float*)p.w;
+    const DnGroup gr = dn_group(p);
+    const int m0 = gr.rbeg + blockIdx.y * TF_M, n0 = blockIdx.x * TF_N;
+    if (m0 >= gr.rend) return;
+    const float* X = (const float*)p.x + gr.xo;
+    const float* W = (const float*)p.w + gr.wo;
+    const float* Bi = p.bias ? (const float*)p.bias + gr.bo : nullptr;
     float acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
     const int lr = tid >> 2, lk = (tid & 3) * 4;          // staging: row lr, k offset lk
-    f32x4 ra = dn_chunk_f32(X, m0 + lr, p.M, lk, p.K, p.ldx, p.vec);
+    const int arow = m0 + lr < gr.rend ? (p.gather ? p.gather[m0 + lr] : m0 + lr) : 0x7fffffff;
+    f32x4 ra = dn_chunk_f32(X, arow, 0x7fffffff, lk, p.K, p.ldx, p.vec);
     f32x4 rb = dn_chunk_f32(W, n0 + lr, p.N, lk, p.K, p.K, p.vec);
     for (int k0 = 0; k0 < p.K; k0 += TF_K) {
         __syncthreads();
@@ -167,7 +196,7 @@ __global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
         for (int i = 0; i < 4; ++i) { As[(lk + i) * TF_LD + lr] = ra[i]; Bs[(lk + i) * TF_LD + lr] = rb[i]; }
         __syncthreads();
         if (k0 + TF_K < p.K) {
-            ra = dn_chunk_f32(X, m0 + lr, p.M, k0 + TF_K + lk, p.K, p.ldx, p.vec);
+            ra = dn_chunk_f32(X, arow, 0x7fffffff, k0 + TF_K + lk, p.K, p.ldx, p.vec);
             rb = dn_chunk_f32(W, n0 + lr, p.N, k0 + TF_K + lk, p.K, p.K, p.vec);
         }
 #pragma unroll
@@ -186,23 +215,23 @@ __global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = m0 + ty * 4 + i;
-        if (row >= p.M) continue;
+        if (row >= gr.rend) continue;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int n = n0 + 2 * tx + j;
             if (p.gated) {
                 if (n + 32 >= p.N) continue;
                 float g = acc[i][j], u = acc[i][j + 2];
-                if (p.bias) { g += ((const float*)p.bias)[n]; u += ((const float*)p.bias)[n + 32]; }
-                dn_store<float>(p, row, (n >> 6) * 32 + (n & 31), dn_act(g, p.act) * u);
+                if (Bi) { g += Bi[n]; u += Bi[n + 32]; }
+                dn_store<float>(p, row, (int)gr.yo + (n >> 6) * 32 + (n & 31), dn_act(g, p.act) * u);
             } else {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
                     const int nn = n + 32 * h;
                     if (nn >= p.N) continue;
                     float v = acc[i][j + 2 * h];
-                    if (p.bias) v += ((const float*)p.bias)[nn];
-                    dn_store<float>(p, row, nn, dn_act(v, p.act));
+                    if (Bi) v += Bi[nn];
+                    dn_store<float>(p, row, (int)gr.yo + nn, dn_act(v, p.act));
                 }
             }
         }
@@ -390,6 +419,7 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
     p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr;
     (void)es;
     hipStream_t st = (hipStream_t)stream;
     if (bf && M > 1 && M <= 16 && p.vec) {
@@ -412,6 +442,40 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
         MI355_CHECK_LAUNCH("dense_tile_bf16_kernel");
     } else {
         const dim3 grid((N + TF_N - 1) / TF_N, (M + TF_M - 1) / TF_M);
+        hipLaunchKernelGGL(dense_tile_f32_kernel, grid, dim3(256), 0, st, p);
+        MI355_CHECK_LAUNCH("dense_tile_f32_kernel");
+    }
+    return MI355_OK;
+}
+
+// The same product for G groups in one launch (tile kernels at every M): group g uses the weight w + g * N * K ([G, N, K] contiguous) and
+// bias + g * N, reads x from column xs * g on and writes y from column ys * g on.  offs null: every group takes all M rows (per-head
+// projections: xs, ys = the head's column step).  offs [G + 1] (device): M rows are sorted by group, group g owns rows offs[g] .. offs[g + 1] - 1;
+// sorted row r reads x row gather[r] (device, or null for r itself) and writes y row r (experts of a mixture: xs = ys = 0).  A row's result
+// depends on its own input and its group's weight only.
+extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y,
+                                   int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs,
+                                   int64_t ys, const int32_t* offs, const int32_t* gather, mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && G > 0 && xs >= 0 && ys >= 0, "dense_grouped: M=%d N=%d K=%d G=%d", M, N, K, G);
+    MI355_CHECK_ARG(ldx >= xs * (G - 1) + K, "dense_grouped: ldx=%d for %d groups of K=%d at step %lld", ldx, G, K, (long long)xs);
+    MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_grouped: act_dtype=%d (bf16 or fp32)", act_dtype);
+    MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_grouped: gated needs N %% 64 == 0 (N=%d)", N);
+    MI355_CHECK_ARG(act >= 0 && act <= 2, "dense_grouped: act=%d", act);
+    MI355_CHECK_ARG(ldy >= ys * (G - 1) + (gated ? N / 2 : N), "dense_grouped: ldy=%d", ldy);
+    MI355_CHECK_ARG(G <= 65535 && (!gather || offs), "dense_grouped: G=%d, gather needs offs", G);
+    const bool bf = act_dtype == MI355_ACT_BF16;
+    DenseParams p;
+    p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
+    p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = 0.f;
+    p.vec = (K % 8 == 0) && (ldx % 8 == 0) && (xs % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+    p.G = G; p.xs = xs; p.ws = (long long)N * K; p.ys = ys; p.offs = offs; p.gather = gather;
+    hipStream_t st = (hipStream_t)stream;
+    if (bf) {
+        const dim3 grid((N + TB_N - 1) / TB_N, (M + TB_M - 1) / TB_M, G);
+        hipLaunchKernelGGL(dense_tile_bf16_kernel, grid, dim3(256), 0, st, p);
+        MI355_CHECK_LAUNCH("dense_tile_bf16_kernel");
+    } else {
+        const dim3 grid((N + TF_N - 1) / TF_N, (M + TF_M - 1) / TF_M, G);
         hipLaunchKernelGGL(dense_tile_f32_kernel, grid, dim3(256), 0, st, p);
         MI355_CHECK_LAUNCH("dense_tile_f32_kernel");
     }

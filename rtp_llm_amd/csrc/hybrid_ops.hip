@@ -57,11 +57,12 @@ template <typename T> __device__ __forceinline__ void hy_store4(T* p, const floa
 template <> __device__ __forceinline__ void hy_store4<float>(float* p, const float (&o)[4]) { *(f32x4*)p = f32x4{o[0], o[1], o[2], o[3]}; }
 template <> __device__ __forceinline__ void hy_store4<bf16>(bf16* p, const float (&o)[4]) { *(u32x2*)p = u32x2{act_pack<true>(o[0], o[1]), act_pack<true>(o[2], o[3])}; }
 
-// x[src] <- x[src] + mult * (a[src] + b[src]) (written back unless rows are gathered), then h1 = norm(x) * (off + w1), h2 likewise.
+// x[src] <- x[src] + mult * (ga * a[src] + gb * b[src]) (written back unless rows are gathered), then h1 = norm(x) * (off + w1), h2 likewise.
+// gate null: ga = gb = 1; else ga = sigmoid(gate[src, c]) and gb = sigmoid(gate[src, W + c]) (fp32 pre-activations, row stride ldg).
 // VEC: W % 4 == 0, four channels per thread and trip (16-byte accesses on the fp32 stream).
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, float mult, const int32_t* rows,
-                                                               const T* w1, const T* w2, float off, float eps, int W, T* h1, T* h2) {
+__global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, const float* gate, int ldg, float mult,
+                                                               const int32_t* rows, const T* w1, const T* w2, float off, float eps, int W, T* h1, T* h2) {
     extern __shared__ __attribute__((aligned(16))) float hy_xs[];
     __shared__ float red[4];
     const int r = blockIdx.x, src = rows ? rows[r] : r;
@@ -72,6 +73,14 @@ __global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const f
         float v[4], ya[4] = {0.f, 0.f, 0.f, 0.f}, yb[4] = {0.f, 0.f, 0.f, 0.f};
         if (VEC) { hy_load4<float>(x + i, v); if (a) hy_load4<float>(a + i, ya); if (b) hy_load4<float>(b + i, yb); }
         else     { v[0] = x[i]; if (a) ya[0] = a[i]; if (b) yb[0] = b[i]; }
+        if (gate && (a || b)) {
+            float ga[4] = {0.f, 0.f, 0.f, 0.f}, gb[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* gp = gate + (size_t)src * ldg + c;
+            if (VEC) { if (a) hy_load4<float>(gp, ga); if (b) hy_load4<float>(gp + W, gb); }
+            else     { if (a) ga[0] = gp[0]; if (b) gb[0] = gp[W]; }
+#pragma unroll
+            for (int e = 0; e < V; ++e) { ya[e] *= hy_sigmoid(ga[e]); yb[e] *= hy_sigmoid(gb[e]); }
+        }
         if (a || b) {
 #pragma unroll
             for (int e = 0; e < V; ++e) v[e] = v[e] + mult * (ya[e] + yb[e]);
@@ -109,6 +118,7 @@ struct AttnGeom {
     int rot_dims, rot_layout;     // rotary span of q / k heads (0 = none) and its pair layout
     int v_layout;                 // pair layout of the value rotation
     int page, max_blocks, num_pages;
+    int v_ld;                     // row stride of the value cache in elements (vdim, or wider when the value rows are a part of wider rows)
 };
 
 template <typename T>
@@ -153,7 +163,7 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
     const int lane = tid & 63, wave = tid >> 6;
     for (int head = wave; head < g.G; head += 4) {
         const float* v = row + voff + head * g.vdim;
-        T* vd = vcache + (slot + (size_t)head * g.page) * g.vdim;
+        T* vd = vcache + (slot + (size_t)head * g.page) * g.v_ld;
         float inv = 1.f;
         if (v_norm) {
             float ss = 0.f;
@@ -184,7 +194,7 @@ constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
 __device__ __forceinline__ float hy_lane_f(float v, int j) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), j)); }
 
 template <typename T>
-__global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+__global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const T* kcache, const T* vcache, T* out) {
     constexpr int NV = HY_MAX_VDIM / 64;
@@ -199,14 +209,14 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     for (int d = tid; d < g.dim; d += NT) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
     __syncthreads();
     const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
-    // the sink is a key of score 0 that carries no value: wave 0 starts from m = 0, l = 1
-    float m = (sink && wave == 0) ? 0.f : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
+    // the sink is a key of (unscaled) score sink[h] that carries no value: wave 0 starts from m = sink[h], l = 1
+    float m = (sink && wave == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
     float acc[NV], facc[8];
 #pragma unroll
     for (int i = 0; i < NV; ++i) acc[i] = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) facc[i] = 0.f;
-    const bool fast = g.vdim % 8 == 0;
+    const bool fast = g.vdim % 8 == 0 && g.v_ld % 8 == 0;
     const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 256: KPI >= 2)
     const int grp = lane / LPK, cl = (lane % LPK) * 8;
     const bool gok = grp < KPI;
@@ -256,7 +266,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
                     const float pk = __shfl(pj, kk & 63, 64);
                     const int rk = __shfl(rowi, kk & 63, 64);
                     pw[u] = ok ? pk : 0.f;
-                    if (ok) hy_load8<T>(vcache + (size_t)rk * g.vdim + cl, vv[u]);
+                    if (ok) hy_load8<T>(vcache + (size_t)rk * g.v_ld + cl, vv[u]);
                     else {
 #pragma unroll
                         for (int i = 0; i < 8; ++i) vv[u][i] = 0.f;
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
                 float a = acc[i] * corr;
                 for (int j = 0; j < nv; ++j) {
                     const float pw = hy_lane_f(pj, j);
-                    const size_t vr = (size_t)__builtin_amdgcn_readlane(rowi, j) * g.vdim;
+                    const size_t vr = (size_t)__builtin_amdgcn_readlane(rowi, j) * g.v_ld;
                     a = __builtin_fmaf(pw, cok ? (float)vcache[vr + c] : 0.f, a);
                 }
                 acc[i] = a;
@@ -352,7 +362,7 @@ __device__ __forceinline__ float hy_sum16(float v) {
 constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 80 bytes, 16-byte aligned
 
 template <int DKM, int NCBM, int NWV>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds; waves per block
-__global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, int sink, const float* vfreq,
+__global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
                                                            const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
                                                            bf16* out) {
@@ -387,7 +397,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     float m[4], l[4];
     f32x4 o[NCBM];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { m[e] = sink ? 0.f : -INFINITY; l[e] = (sink && lr == 0) ? 1.f : 0.f; }   // l: per-lane share of the row's denominator
+    for (int e = 0; e < 4; ++e) { m[e] = sink ? sink[h] * 1.44269504088896340736f : -INFINITY; l[e] = (sink && lr == 0) ? 1.f : 0.f; }   // l: per-lane share of the row's denominator
 #pragma unroll
     for (int cb = 0; cb < NCBM; ++cb) o[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int plast = p0 + n - 1;
@@ -412,7 +422,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
             const int i = threadIdx.x + e * 64 * NWV;
             if (i < 32 * VP) {
                 const int kc = min(t0 + (i & 31), plast);
-                vn[e] = *(const u32x4*)(vcache + cache_row(kc) * g.vdim + (i >> 5) * 8);
+                vn[e] = *(const u32x4*)(vcache + cache_row(kc) * g.v_ld + (i >> 5) * 8);
             }
         }
     };
@@ -524,7 +534,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
 // at a time: all threads compute the gates of the staged tokens once into LDS, then every thread walks the tokens in order (its RD rows:
 // decay, rank-one update, partial q . S), and the DS partial outputs per token are summed from LDS.  Short RD keeps the dependent chain per
 // token short; the walk itself is the sequential part of the recurrence.
-enum { SCAN_HGRN2 = 0, SCAN_GLA = 1 };
+enum { SCAN_HGRN2 = 0, SCAN_GLA = 1, SCAN_FIXED = 2 };
 
 struct ScanParams {
     const float* proj; int ld; int qo, ko, vo;     // fp32 projections [rows, ld]: q, k (GLA) or forget pre-activation (HGRN2), v at these columns
@@ -594,7 +604,9 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
             float qv = 0.f, kv = 0.f, av = 1.f;
             if (d < p.dim) {
                 const int hd = h * p.dim + d;
-                if (p.mode == SCAN_HGRN2) {
+                if (p.mode == SCAN_FIXED) {          // one decay per head (fp32 [H] behind `lower`), q and k as given
+                    qv = rq[e]; kv = rk[e]; av = ((const float*)p.lower)[h];
+                } else if (p.mode == SCAN_HGRN2) {
                     const float lw = (float)((const T*)p.lower)[hd];
                     const float f = lw + (1.f - lw) * hy_sigmoid(rk[e] + (float)((const T*)p.fbias)[hd]);
                     qv = hy_silu(rq[e]); av = f; kv = 1.f - f;
@@ -651,7 +663,7 @@ __global__ __launch_bounds__(1024) void hy_scan_kernel(ScanParams p) {
     }
 }
 
-// per-head RMS norm over vdim with a plain weight shared by the heads, optional silu gate: one wave per (row, head)
+// per-head RMS norm over vdim with a plain weight shared by the heads (null: none), optional silu gate: one wave per (row, head)
 template <typename T>
 __global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H, int vdim, const T* w, float eps, const float* gate, int ldg, int goff, T* out) {
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -660,9 +672,241 @@ __global__ __launch_bounds__(64) void hy_head_norm_kernel(const float* o, int H,
     for (int c = lane; c < vdim; c += 64) ss = __builtin_fmaf(src[c], src[c], ss);
     const float inv = 1.f / sqrtf(hy_wave_sum(ss) / (float)vdim + eps);
     for (int c = lane; c < vdim; c += 64) {
-        float v = src[c] * inv * (float)w[c];
+        float v = src[c] * inv;
+        if (w) v *= (float)w[c];
         if (gate) v *= hy_silu(gate[(size_t)r * ldg + goff + h * vdim + c]);
         out[((size_t)r * H + h) * vdim + c] = (T)v;
+    }
+}
+
+
+// ------------------------------------------------------------------------------------------------ latent attention: normed latent + shared rotated key -> page; queries split
+// A token caches ONE row [c (R) | rotated shared key part (dr) | zeros up to dpad] for all heads: c = unit-RMS(first R outputs of the down
+// projection) * w, the key part is the remaining dr outputs with their first `rdims` channels turned by the position (interleaved pairs,
+// cos and sin times `mag`).  Values are the first R channels of the same row.  Per query head the un-rotated part goes to qn (activation
+// type, input of the per-head product with the key up-projection) and the rotated part to columns R.. of the head's absorbed query row
+// (fp32, dpad wide, zeros behind).
+struct LatentGeom { int H, dim, dr, R, dpad, rdims, page, max_blocks, num_pages; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_latent_prep_kernel(const float* proj, int ld, int doff, LatentGeom g, const float* freq, float mag, const T* cw, float eps,
+                                                             const int32_t* pos, const int32_t* seq, const int32_t* block_table, T* qn, float* qabs, T* cache) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int p = pos[r];
+    const float fp = (float)p;
+    const float* row = proj + (size_t)r * ld;
+    const int hd = g.dim + g.dr, hp = g.rdims / 2;
+    // queries
+    for (int i = tid; i < g.H * g.dim; i += 256) qn[(size_t)r * g.H * g.dim + i] = (T)row[(i / g.dim) * hd + i % g.dim];
+    const int tail = g.dpad - g.R;                                   // rotated part + padding of an absorbed query row
+    for (int i = tid; i < g.H * tail; i += 256) {
+        const int h = i / tail, j = i % tail;
+        float v = 0.f;
+        if (j < g.dr) {
+            const float* qr = row + h * hd + g.dim;
+            if (j < g.rdims) {
+                const int pr = j >> 1;
+                float sn, cs;
+                sincosf(fp * freq[pr], &sn, &cs);
+                sn *= mag; cs *= mag;
+                const float u = qr[2 * pr], w = qr[2 * pr + 1];
+                v = (j & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
+            } else v = qr[j];
+        }
+        qabs[((size_t)r * g.H + h) * g.dpad + g.R + j] = v;
+    }
+    (void)hp;
+    // cache row
+    bool ok = p >= 0 && p / g.page < g.max_blocks;
+    int pg = 0;
+    if (ok) { pg = block_table[(size_t)seq[r] * g.max_blocks + p / g.page]; ok = pg >= 0 && pg < g.num_pages; }
+    const float* dk = row + doff;
+    float ss = 0.f;
+    for (int c = tid; c < g.R; c += 256) ss = __builtin_fmaf(dk[c], dk[c], ss);
+    ss = hy_wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    if (!ok) return;
+    const float inv = 1.f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)g.R + eps);
+    T* dst = cache + ((size_t)pg * g.page + (p % g.page)) * g.dpad;
+    for (int c = tid; c < g.dpad; c += 256) {
+        float v = 0.f;
+        if (c < g.R) v = dk[c] * inv * (float)cw[c];
+        else if (c < g.R + g.dr) {
+            const int j = c - g.R;
+            if (j < g.rdims) {
+                const int pr = j >> 1;
+                float sn, cs;
+                sincosf(fp * freq[pr], &sn, &cs);
+                sn *= mag; cs *= mag;
+                const float u = dk[g.R + 2 * pr], w = dk[g.R + 2 * pr + 1];
+                v = (j & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
+            } else v = dk[c];
+        }
+        dst[c] = (T)v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ rotary on fp32 projections, in place
+// Up to two segments of heads in one buffer (queries and keys): the first `rdims` channels of every head are turned by position * freq
+// (pair layout 0 / 1 as hy_pair), cos and sin times `mag`; then the whole head is multiplied by the segment's scale.
+struct RotSeg { int off, heads, dim; float scale; };
+
+__global__ __launch_bounds__(256) void hy_rotary_kernel(float* buf, int ld, RotSeg s0, RotSeg s1, int rdims, int layout, const float* freq, float mag,
+                                                        const int32_t* pos) {
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float fp = (float)pos[r];
+    float* row = buf + (size_t)r * ld;
+    const int hp = rdims / 2;
+    for (int sg = 0; sg < 2; ++sg) {
+        const RotSeg s = sg ? s1 : s0;
+        for (int i = tid; i < s.heads * hp; i += 256) {
+            const int head = i / hp, pr = i % hp;
+            int c0, c1;
+            hy_pair(layout, pr, rdims, c0, c1);
+            float sn, cs;
+            sincosf(fp * freq[pr], &sn, &cs);
+            sn *= mag; cs *= mag;
+            float* b = row + s.off + head * s.dim;
+            const float u = b[c0], v = b[c1];
+            b[c0] = (u * cs - v * sn) * s.scale; b[c1] = (v * cs + u * sn) * s.scale;
+        }
+        if (s.scale != 1.f)
+            for (int i = tid; i < s.heads * (s.dim - rdims); i += 256) {
+                float* b = row + s.off + (i / (s.dim - rdims)) * s.dim + rdims + i % (s.dim - rdims);
+                *b *= s.scale;
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ PolyNorm activation
+// out = a N(z) + b N(z^2) + c N(z^3) + e per row, N(u) = u / sqrt(mean(u^2) + eps) over the row's n channels; z fp32 [rows, ld].
+__device__ __forceinline__ float hy_block_sum3(float& a, float& b, float& c, float (*red)[4]) {
+    a = hy_wave_sum(a); b = hy_wave_sum(b); c = hy_wave_sum(c);
+    if ((threadIdx.x & 63) == 0) { red[0][threadIdx.x >> 6] = a; red[1][threadIdx.x >> 6] = b; red[2][threadIdx.x >> 6] = c; }
+    __syncthreads();
+    a = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+    b = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+    c = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+    return a;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void hy_polynorm_kernel(const float* z, int ld, int n, float ca, float cb, float cc, float ce, float eps, T* out, int ldo) {
+    __shared__ float red[3][4];
+    const int r = blockIdx.x;
+    const float* zr = z + (size_t)r * ld;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float v = zr[c], v2 = v * v, v3 = v2 * v;
+        s1 = __builtin_fmaf(v, v, s1); s2 = __builtin_fmaf(v2, v2, s2); s3 = __builtin_fmaf(v3, v3, s3);
+    }
+    hy_block_sum3(s1, s2, s3, red);
+    const float i1 = ca / sqrtf(s1 / (float)n + eps), i2 = cb / sqrtf(s2 / (float)n + eps), i3 = cc / sqrtf(s3 / (float)n + eps);
+    for (int c = threadIdx.x; c < n; c += 256) {
+        const float v = zr[c], v2 = v * v;
+        out[(size_t)r * ldo + c] = (T)(((v * i1 + v2 * i2) + v2 * v * i3) + ce);
+    }
+}
+
+// out = (T)(o * sigmoid(gate)) elementwise: o fp32 [rows, n], gate fp32 [rows, ldg] from column goff
+template <typename T>
+__global__ __launch_bounds__(256) void hy_gate_mul_kernel(const float* o, int n, const float* gate, int ldg, int goff, T* out) {
+    const int r = blockIdx.x;
+    for (int c = threadIdx.x; c < n; c += 256)
+        out[(size_t)r * n + c] = (T)(o[(size_t)r * n + c] * hy_sigmoid(gate[(size_t)r * ldg + goff + c]));
+}
+
+// ------------------------------------------------------------------------------------------------ mixture of experts: routing, sorting by expert, weighted sum
+// One wave per token: softmax over the E router logits (fp32); experts come in `groups` runs of E / groups neighbours, a group scores as its
+// best expert and only the `keep` best groups stay eligible; the `top` eligible experts with the largest scores are chosen, ties to the lower
+// index; the weights are their softmax scores as they are.
+__device__ __forceinline__ void hy_wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, 64);
+        const int oi = __shfl_xor(i, o, 64);
+        if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+__global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld, int E, int groups, int keep, int top, int32_t* ids, float* wts) {
+    extern __shared__ float hy_rs[];            // scores [E], group best [groups]
+    float* sc = hy_rs;
+    float* gb = hy_rs + E;
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* zr = z + (size_t)t * ld;
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
+    m = hy_wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) { const float x = expf(zr[e] - m); sc[e] = x; sum += x; }
+    sum = hy_wave_sum(sum);
+    for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
+    __syncthreads();
+    const int per = E / groups;
+    if (groups > 1 && keep < groups) {
+        for (int g = lane; g < groups; g += 64) {
+            float b = -1.f;
+            for (int j = 0; j < per; ++j) b = fmaxf(b, sc[g * per + j]);
+            gb[g] = b;
+        }
+        __syncthreads();
+        for (int k = 0; k < keep; ++k) {          // the kept groups get a best score of 2 (above any probability), the others stay below
+            float bv = -2.f; int bi = 0x7fffffff;
+            for (int g = lane; g < groups; g += 64) { const float v = gb[g]; if (v <= 1.5f && (v > bv || (v == bv && g < bi))) { bv = v; bi = g; } }
+            hy_wave_argmax(bv, bi);
+            if (lane == 0) gb[bi] = 2.f;
+            __syncthreads();
+        }
+    } else {
+        for (int g = lane; g < groups; g += 64) gb[g] = 2.f;
+        __syncthreads();
+    }
+    for (int k = 0; k < top; ++k) {
+        float bv = -2.f; int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += 64) {
+            const float v = sc[e];
+            if (v >= 0.f && gb[e / per] > 1.5f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
+        }
+        hy_wave_argmax(bv, bi);
+        if (lane == 0) { ids[(size_t)t * top + k] = bi; wts[(size_t)t * top + k] = bv; sc[bi] = -1.f; }     // taken
+        __syncthreads();
+    }
+}
+
+// Counting sort of the n = tokens * top (token, choice) pairs by expert, one block: offs [E + 1], src_row[sorted place] = token,
+// place_of[pair] = sorted place.  The order inside an expert is arbitrary (rows are independent of each other).
+__global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, int n, int top, int E, int32_t* offs, int32_t* src_row, int32_t* place_of) {
+    extern __shared__ int hy_cnt[];             // counts [E], cursors [E]
+    int* cnt = hy_cnt;
+    int* cur = hy_cnt + E;
+    for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int a = 0;
+        for (int e = 0; e < E; ++e) { cur[e] = a; offs[e] = a; a += cnt[e]; }
+        offs[E] = a;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int at = atomicAdd(&cur[ids[i]], 1);
+        src_row[at] = i / top;
+        place_of[i] = at;
+    }
+}
+
+// out[t] = sum_k wts[t, k] * y[place_of[t * top + k]] (+ extra[t]): fp32 [tokens, W], the choices added in order k = 0 .. top - 1
+__global__ __launch_bounds__(256) void hy_moe_combine_kernel(const float* y, int W, const int32_t* place_of, const float* wts, int top, const float* extra, float* out) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float a = 0.f;
+        for (int k = 0; k < top; ++k) a = __builtin_fmaf(wts[(size_t)t * top + k], y[(size_t)place_of[(size_t)t * top + k] * W + c], a);
+        if (extra) a += extra[(size_t)t * W + c];
+        out[(size_t)t * W + c] = a;
     }
 }
 
@@ -672,6 +916,7 @@ int hy_geom_ok(const AttnGeom& g) {
     MI355_CHECK_ARG(g.vdim > 0 && g.vdim % 2 == 0 && g.vdim <= HY_MAX_VDIM, "hybrid attention: value size %d (even, <= %d)", g.vdim, HY_MAX_VDIM);
     MI355_CHECK_ARG(g.rot_dims >= 0 && g.rot_dims <= g.dim && g.rot_dims % 2 == 0, "hybrid attention: rotary span %d of %d", g.rot_dims, g.dim);
     MI355_CHECK_ARG(g.page > 0 && g.max_blocks > 0 && g.num_pages > 0, "hybrid attention: page=%d max_blocks=%d pages=%d", g.page, g.max_blocks, g.num_pages);
+    MI355_CHECK_ARG(g.v_ld >= g.vdim, "hybrid attention: value row stride %d under the value size %d", g.v_ld, g.vdim);
     MI355_CHECK_ARG((long long)g.num_pages * g.G * g.page < (1ll << 31), "hybrid attention: %d pages x %d heads x %d tokens overflow a 32-bit row index", g.num_pages, g.G, g.page);
     return MI355_OK;
 }
@@ -695,20 +940,28 @@ extern "C" int mi355_hy_embed(const int32_t* ids, int32_t rows, const void* tabl
 
 // x [*, W] fp32 stream; a, b [*, W] fp32 branch outputs (either may be null); rows: null, or `n` source rows to gather (x is then read only).
 // h1 / h2 [n, W] of act_dtype: x / rms(x) * (weight_offset + w).  w2 / h2 may be null.
+// gate: null, or fp32 [*, ldg] pre-activations of per-channel branch gates: a is scaled by sigmoid(gate[:, 0:W]), b by sigmoid(gate[:, W:2W]).
+extern "C" int mi355_hy_gated_residual_norm(float* x, const float* a, const float* b, const float* gate, int32_t ldg, float mult, const int32_t* rows,
+                                            int32_t n, int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2,
+                                            int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(x && n > 0 && W > 0 && (!h1 || w1) && (!h2 || w2), "hy_residual_norm: n=%d W=%d", n, W);
+    MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_residual_norm: W=%d too wide for one block", W);
+    MI355_CHECK_ARG(!gate || ldg >= 2 * W, "hy_residual_norm: gate row stride %d for two gates of %d", ldg, W);
+    auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
+    if (W % 4 == 0 && ldg % 4 == 0 && al(x) && al(a) && al(b) && al(gate) && al(w1) && al(w2) && al(h1) && al(h2))
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, gate, ldg,
+                                                  mult, rows, (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
+    else
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, gate, ldg,
+                                                  mult, rows, (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
+    MI355_CHECK_LAUNCH("hy_residual_norm_kernel");
+    return MI355_OK;
+}
+
 extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, float mult, const int32_t* rows, int32_t n, int32_t W,
                                       const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
                                       mi355_stream_t stream) {
-    MI355_CHECK_ARG(x && n > 0 && W > 0 && (!h1 || w1) && (!h2 || w2), "hy_residual_norm: n=%d W=%d", n, W);
-    MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_residual_norm: W=%d too wide for one block", W);
-    auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
-    if (W % 4 == 0 && al(x) && al(a) && al(b) && al(w1) && al(w2) && al(h1) && al(h2))
-        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
-                                                  (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
-    else
-        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, mult, rows,
-                                                  (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
-    MI355_CHECK_LAUNCH("hy_residual_norm_kernel");
-    return MI355_OK;
+    return mi355_hy_gated_residual_norm(x, a, b, nullptr, 0, mult, rows, n, W, w1, w2, weight_offset, eps, h1, h2, act_dtype, stream);
 }
 
 // geom: {H, G, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages}.  qkv fp32 [rows, ld]: q heads at column 0 (rotated in
@@ -718,7 +971,7 @@ extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t 
                                   int32_t v_norm, float eps, const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows,
                                   void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(qkv && geom && pos && seq && rows > 0, "hy_attn_prep: null argument");
-    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     MI355_CHECK_ARG((g.rot_dims == 0 || kfreq) && (!kcache || (vcache && block_table)), "hy_attn_prep: missing table or cache");
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_prep_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, qkv, ld, koff, voff, g, kfreq, vfreq,
@@ -728,12 +981,12 @@ extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t 
 }
 
 // out [rows, H * vdim] of act_dtype.  chunk > 0: row at position i sees keys j <= i of its own block of `chunk` positions; 0: all j <= i.
-// sink: one is added to the softmax denominator.  vfreq non-null: the head output is turned back by the row's position.
-extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+// sink: null, or fp32 [H]: exp(sink[h]) is added to head h's softmax denominator (a key of that unscaled score without a value).  vfreq non-null: the head output is turned back by the row's position.
+extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                                   const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
                                   const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
-    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     const int threads = rows * g.H <= 2048 ? 1024 : 256;     // few (decode) rows: sixteen waves share a row's keys
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(threads), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
@@ -744,14 +997,14 @@ extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, cons
 
 // The same attention for prompt portions (bf16 cache): tile t covers rows tile_row0[t] .. + tile_n[t] - 1 (<= 16, consecutive positions of one
 // sequence).  Needs dim % 32 == 0 and vdim % 16 == 0 (% 32 under the halves layout), both <= 256: MI355_ERR_UNSUPPORTED otherwise.
-extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, int32_t sink, const float* vfreq,
+extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                                    const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0,
                                    const int32_t* tile_n, int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype,
                                    mi355_stream_t stream) {
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && tile_row0 && tile_n && kcache && vcache && out && tiles > 0 && chunk >= 0, "hy_attn_tiles: bad argument");
-    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9]};
+    const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
-    if (act_dtype != MI355_ACT_BF16 || g.dim % 32 || g.dim > 256 || g.vdim % 16 || g.vdim > 256 || (vfreq && g.v_layout != 0 && g.vdim % 32)) {
+    if (act_dtype != MI355_ACT_BF16 || g.dim % 32 || g.dim > 256 || g.vdim % 16 || g.vdim > 256 || g.v_ld % 8 || (vfreq && g.v_layout != 0 && g.vdim % 32)) {
         mi355_set_error("hy_attn_tiles: bf16, dim %% 32 == 0, vdim %% 16 == 0 only (dim=%d vdim=%d dtype=%d)", g.dim, g.vdim, act_dtype);
         return MI355_ERR_UNSUPPORTED;
     }
@@ -768,6 +1021,7 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
 
 // mode 0 (HGRN2): q = silu(proj q), f = lower + (1 - lower) sigmoid(proj k + fbias), a = f, k = 1 - f.
 // mode 1 (GLA):   q = proj q * qscale, k = proj k, a = sigmoid(z)^(1 / tau).
+// mode 2 (fixed): q = proj q, k = proj k, a = lower[h] (fp32 [H], one decay per head whatever act_dtype is).
 // Sequence s owns rows row_start[s] .. row_start[s + 1] - 1 in order, continues the state in slot[s] (starts from zero when first_pos[s] == 0)
 // and leaves the new state there.  out fp32 [rows, H * vdim].
 extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_t qo, int32_t ko, int32_t vo, const float* z, int32_t ldz,
@@ -775,7 +1029,8 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
                              const int32_t* row_start, const int32_t* slot, const int32_t* first_pos, int32_t nseq, float* state, float* out,
                              int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(proj && row_start && slot && first_pos && state && out && nseq > 0 && H > 0 && dim > 0 && vdim > 0, "hy_scan: bad argument");
-    MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : (mode == SCAN_GLA && z && tau > 0.f), "hy_scan: mode %d lacks its gate inputs", mode);
+    MI355_CHECK_ARG(mode == SCAN_HGRN2 ? (lower && fbias) : mode == SCAN_FIXED ? lower != nullptr : (mode == SCAN_GLA && z && tau > 0.f),
+                    "hy_scan: mode %d lacks its gate inputs", mode);
     MI355_CHECK_ARG(dim <= 512, "hy_scan: key size %d > 512", dim);
     const int RD = dim <= 128 ? 8 : dim <= 256 ? 16 : 32;       // rows per thread: at most 16 groups of RD rows (1024 threads)
     const int DS = (dim + RD - 1) / RD;
@@ -794,9 +1049,81 @@ extern "C" int mi355_hy_scan(int32_t mode, const float* proj, int32_t ld, int32_
 
 extern "C" int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, const void* w, float eps, const float* gate, int32_t ldg,
                                   int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream) {
-    MI355_CHECK_ARG(o && w && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
+    MI355_CHECK_ARG(o && out && rows > 0 && H > 0 && vdim > 0, "hy_head_norm: bad argument");
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_head_norm_kernel<T>, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, o, H, vdim, (const T*)w, eps, gate, ldg,
                                               goff, (T*)out));
     MI355_CHECK_LAUNCH("hy_head_norm_kernel");
+    return MI355_OK;
+}
+
+// geom: {H, dim, dr, R, dpad, rdims, page, max_blocks, num_pages}.  proj fp32 [rows, ld]: H query heads of dim + dr channels from column 0, the down
+// projection (R + dr channels) from column doff.  freq [rdims / 2] fp32, mag multiplies cos and sin; cw [R] norm weight of act_dtype.
+// qn [rows, H * dim] act_dtype, qabs fp32 [rows, H * dpad] (columns R .. dpad - 1 of every head are written), cache [pages, page, dpad] act_dtype.
+extern "C" int mi355_hy_latent_prep(const float* proj, int32_t ld, int32_t doff, const int32_t* geom, const float* freq, float mag, const void* cw, float eps,
+                                    const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, void* qn, float* qabs, void* cache,
+                                    int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(proj && geom && cw && pos && seq && block_table && qn && qabs && cache && rows > 0, "hy_latent_prep: null argument");
+    const LatentGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8]};
+    MI355_CHECK_ARG(g.H > 0 && g.dim > 0 && g.dr >= 0 && g.R > 0 && g.dpad >= g.R + g.dr && g.rdims >= 0 && g.rdims <= g.dr && g.rdims % 2 == 0 && (g.rdims == 0 || freq),
+                    "hy_latent_prep: heads=%d dim=%d rot=%d rank=%d padded=%d span=%d", g.H, g.dim, g.dr, g.R, g.dpad, g.rdims);
+    MI355_CHECK_ARG(g.page > 0 && g.max_blocks > 0 && g.num_pages > 0 && ld >= doff + g.R + g.dr && doff >= g.H * (g.dim + g.dr), "hy_latent_prep: ld=%d doff=%d", ld, doff);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_latent_prep_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, proj, ld, doff, g, freq, mag, (const T*)cw, eps,
+                                              pos, seq, block_table, (T*)qn, qabs, (T*)cache));
+    MI355_CHECK_LAUNCH("hy_latent_prep_kernel");
+    return MI355_OK;
+}
+
+// buf fp32 [rows, ld]; segment i: heads_i heads of dim_i channels from column off_i, multiplied by scale_i after the turn (heads1 = 0: one segment).
+extern "C" int mi355_hy_rotary(float* buf, int32_t ld, int32_t rows, int32_t off0, int32_t heads0, int32_t dim0, float scale0, int32_t off1, int32_t heads1,
+                               int32_t dim1, float scale1, int32_t rdims, int32_t layout, const float* freq, float mag, const int32_t* pos, mi355_stream_t stream) {
+    MI355_CHECK_ARG(buf && pos && rows > 0 && rdims >= 0 && rdims % 2 == 0 && (rdims == 0 || freq) && (layout == 0 || layout == 1), "hy_rotary: bad argument");
+    MI355_CHECK_ARG(heads0 >= 0 && heads1 >= 0 && (heads0 == 0 || rdims <= dim0) && (heads1 == 0 || rdims <= dim1), "hy_rotary: span %d of heads of %d / %d", rdims, dim0, dim1);
+    MI355_CHECK_ARG(off0 + heads0 * dim0 <= ld && off1 + heads1 * dim1 <= ld, "hy_rotary: segments past the row (ld=%d)", ld);
+    hipLaunchKernelGGL(hy_rotary_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, buf, ld, RotSeg{off0, heads0, dim0, scale0}, RotSeg{off1, heads1, dim1, scale1},
+                       rdims, layout, freq, mag, pos);
+    MI355_CHECK_LAUNCH("hy_rotary_kernel");
+    return MI355_OK;
+}
+
+extern "C" int mi355_hy_polynorm(const float* z, int32_t ld, int32_t rows, int32_t n, float ca, float cb, float cc, float ce, float eps, void* out, int32_t ldo,
+                                 int32_t act_dtype, mi355_stream_t stream) {
+    MI355_CHECK_ARG(z && out && rows > 0 && n > 0 && ld >= n && ldo >= n, "hy_polynorm: rows=%d n=%d", rows, n);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_polynorm_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, z, ld, n, ca, cb, cc, ce, eps, (T*)out, ldo));
+    MI355_CHECK_LAUNCH("hy_polynorm_kernel");
+    return MI355_OK;
+}
+
+extern "C" int mi355_hy_gate_mul(const float* o, int32_t rows, int32_t n, const float* gate, int32_t ldg, int32_t goff, void* out, int32_t act_dtype,
+                                 mi355_stream_t stream) {
+    MI355_CHECK_ARG(o && gate && out && rows > 0 && n > 0 && goff >= 0 && ldg >= goff + n, "hy_gate_mul: rows=%d n=%d", rows, n);
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_gate_mul_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, o, n, gate, ldg, goff, (T*)out));
+    MI355_CHECK_LAUNCH("hy_gate_mul_kernel");
+    return MI355_OK;
+}
+
+// z fp32 [tokens, ld] router logits -> ids int32 [tokens, top], wts fp32 [tokens, top]
+extern "C" int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                                  mi355_stream_t stream) {
+    MI355_CHECK_ARG(z && ids && wts && tokens > 0 && E > 0 && ld >= E, "hy_moe_route: tokens=%d experts=%d", tokens, E);
+    MI355_CHECK_ARG(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= (E / groups) * keep, "hy_moe_route: %d experts in %d groups, keep %d, top %d",
+                    E, groups, keep, top);
+    MI355_CHECK_ARG((size_t)(E + groups) * 4 <= 48 * 1024, "hy_moe_route: %d experts do not fit the block's scratch", E);
+    hipLaunchKernelGGL(hy_moe_route_kernel, dim3(tokens), dim3(64), (size_t)(E + groups) * 4, (hipStream_t)stream, z, ld, E, groups, keep, top, ids, wts);
+    MI355_CHECK_LAUNCH("hy_moe_route_kernel");
+    return MI355_OK;
+}
+
+extern "C" int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, int32_t E, int32_t* offs, int32_t* src_row, int32_t* place_of, mi355_stream_t stream) {
+    MI355_CHECK_ARG(ids && offs && src_row && place_of && n > 0 && top > 0 && E > 0 && (size_t)E * 8 <= 48 * 1024, "hy_moe_align: n=%d experts=%d", n, E);
+    hipLaunchKernelGGL(hy_moe_align_kernel, dim3(1), dim3(1024), (size_t)E * 8, (hipStream_t)stream, ids, n, top, E, offs, src_row, place_of);
+    MI355_CHECK_LAUNCH("hy_moe_align_kernel");
+    return MI355_OK;
+}
+
+extern "C" int mi355_hy_moe_combine(const float* y, int32_t tokens, int32_t W, const int32_t* place_of, const float* wts, int32_t top, const float* extra, float* out,
+                                    mi355_stream_t stream) {
+    MI355_CHECK_ARG(y && place_of && wts && out && tokens > 0 && W > 0 && top > 0, "hy_moe_combine: tokens=%d W=%d", tokens, W);
+    hipLaunchKernelGGL(hy_moe_combine_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, y, W, place_of, wts, top, extra, out);
+    MI355_CHECK_LAUNCH("hy_moe_combine_kernel");
     return MI355_OK;
 }

@@ -1,13 +1,17 @@
-"""The hybrid decoder family: a stack of parallel-residual layers  x <- x + m * (mixer(norm1 x) + mlp(norm2 x))  over an fp32 residual
-stream, every layer with its own mixer (mixers.PagedChunkAttention or mixers.GatedLinearRecurrence) and an optional gated MLP, a final
-norm, the output head and an optional tanh soft cap of the logits.  Norm weights are stored as offsets from one.
+"""The hybrid decoder family: a stack of parallel-residual layers  x <- x + m * (g1 * mixer(norm1 x) + g2 * mlp(norm2 x))  over an fp32
+residual stream, every layer with its own mixer (mixers.PagedChunkAttention, GatedLinearRecurrence, LatentAttention or Retention) and an
+optional feed-forward (gated dense, PolyNorm dense, or routed experts), a final norm, the output head and an optional tanh soft cap of the
+logits.  Per member of the family: norm weights stored as offsets from one or plain; one norm per branch or one for both; branch gates
+g = sigmoid(W h + b) per channel or none.
 
 ``HybridConfig.from_json`` reads the family's config.json (keys: architecture, vocab, width, residual_mult, logit_softcap, norm.eps and
 layers[i].{type, mixer, mlp}); ``HybridModel`` holds the device weights (checkpoint tensors embed, l<i>.norm1/2, l<i>.mix.*, l<i>.mlp.*,
 final.norm, head) and runs one ragged step against the cache tensors an engine allocated from ``cache_layout()``.
 
-Nufalorn is the member of the family registered here: chunk-masked sink attention with unit-normed, rotated values and shared-KV
-layers, HGRN2 and GLA recurrences, relu-gated MLPs."""
+Members: Nufalorn (chunk-masked sink attention with unit-normed, rotated values and shared-KV layers, HGRN2 and GLA recurrences,
+relu-gated MLPs, two offset norms per layer) and Pokepel (latent attention and retention, PolyNorm MLPs and group-limited mixtures of
+silu-gated experts with a shared expert, one plain norm per layer, sigmoid-gated branches; checkpoint tensors l<i>.rg1 / rg2 (+ .b),
+l<i>.mlp.{up, down, act} or l<i>.mlp.{router, e<j>.{gate, up, down}, shared.{gate, up, down}})."""
 import json
 import os
 from dataclasses import dataclass, field
@@ -16,15 +20,19 @@ from typing import Dict, List, Optional, Union
 import torch
 
 from . import hybrid_ops as hops
-from .mixers import AttentionSpec, GatedLinearRecurrence, GatedMLP, PagedChunkAttention, RecurrenceSpec, RotarySpec, StepBatch
+from .mixers import (AttentionSpec, GatedLinearRecurrence, GatedMLP, LatentAttention, LatentAttentionSpec, PagedChunkAttention, PolyNormMLP,
+                     RecurrenceSpec, Retention, RetentionSpec, RotarySpec, RoutedExperts, RouterSpec, StepBatch)
 
 
 @dataclass
 class HybridLayerSpec:
-    kind: str                                        # "attention" | "hgrn2" | "gla"
-    mixer: Union[AttentionSpec, RecurrenceSpec]
-    ff: Optional[int] = None                         # None: the layer has no MLP
+    kind: str                                        # "attention" | "hgrn2" | "gla" | "latent_attention" | "retention"
+    mixer: Union[AttentionSpec, RecurrenceSpec, LatentAttentionSpec, RetentionSpec]
+    ff: Optional[int] = None                         # None: the layer has no MLP; hidden size of the dense MLP or of one routed expert
     mlp_act: str = "relu"
+    mlp_kind: str = "gated"                          # "gated" | "polynorm" | "experts"
+    router: Optional[RouterSpec] = None              # experts: the router ...
+    shared_ff: Optional[int] = None                  # ... and the hidden size of the expert every token runs (None: no such expert)
 
 
 @dataclass
@@ -37,9 +45,19 @@ class HybridConfig:
     residual_mult: float = 1.0
     logit_softcap: float = 0.0
     norm_offset: float = 1.0                         # stored norm weights are offsets from this value
+    shared_norm: bool = False                        # one norm per layer feeds the mixer and the MLP
+    branch_gates: bool = False                       # each branch is multiplied by sigmoid(W h + b) of its input before it joins the stream
 
     @staticmethod
     def from_json(cfg: dict) -> "HybridConfig":
+        """config.json -> the configuration of the member its "architecture" names."""
+        reader = _READERS.get(str(cfg.get("architecture", "")).lower())
+        if reader is None:
+            raise NotImplementedError(f"hybrid family: architecture {cfg.get('architecture')!r} (known: {', '.join(sorted(_READERS))})")
+        return reader(cfg)
+
+    @staticmethod
+    def nufalorn_from_json(cfg: dict) -> "HybridConfig":
         """The Nufalorn reading of config.json: attention layers have the softmax sink, unit-normed values and values rotated in the key
         layout (interleaved pairs); MLPs are relu-gated; norm weights are stored around zero."""
         layers = []
@@ -70,6 +88,44 @@ class HybridConfig:
                             eps=float(cfg["norm"]["eps"]), residual_mult=float(cfg.get("residual_mult", 1.0)),
                             logit_softcap=float(cfg.get("logit_softcap") or 0.0))
 
+    @staticmethod
+    def pokepel_from_json(cfg: dict) -> "HybridConfig":
+        """The Pokepel reading of config.json: latent attention (interleaved rotary pairs on the rotated part, optional YaRN scaling, learned
+        sink, output gate) and retention (rotary pairs half a span apart, one decay per head); dense MLPs use PolyNorm, mixtures have silu-gated
+        experts; one plain norm per layer, gated branches, no residual multiplier or soft cap."""
+        layers = []
+        for i, L in enumerate(cfg["layers"]):
+            kind, mx, mlp = L["type"], L["mixer"], L.get("mlp")
+            if kind == "latent_attention":
+                rot = dict(mx.get("rot") or {})
+                rot.setdefault("dims", mx["rot_dim"])
+                spec = LatentAttentionSpec(heads=int(mx["heads"]), dim=int(mx["dim"]), rot_dim=int(mx["rot_dim"]), vdim=int(mx["vdim"]),
+                                           kv_rank=int(mx["kv_rank"]), scale=float(mx["scale"]),
+                                           rot=RotarySpec.from_json(rot if "base" in rot else None, "interleaved"))
+            elif kind == "retention":
+                if len(mx["decay"]) != int(mx["heads"]):
+                    raise ValueError(f"layer {i}: {len(mx['decay'])} decays for {mx['heads']} heads")
+                spec = RetentionSpec(heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx["vdim"]), decay=tuple(float(a) for a in mx["decay"]),
+                                     rot=RotarySpec.from_json(mx.get("rot"), "halves"))
+            else:
+                raise NotImplementedError(f"layer {i}: mixer type {kind!r}")
+            if mlp is None:
+                layers.append(HybridLayerSpec(kind, spec))
+            elif mlp.get("kind", "dense") == "dense":
+                layers.append(HybridLayerSpec(kind, spec, int(mlp["ff"]), "polynorm", "polynorm"))
+            elif mlp["kind"] == "moe":
+                r, grp, sh = mlp["router"], mlp["router"].get("groups") or {}, mlp.get("shared")
+                layers.append(HybridLayerSpec(kind, spec, int(mlp["expert"]["ff"]), "silu", "experts",
+                                              RouterSpec(int(r["experts"]), int(r["top"]), int(grp.get("count", 1)), int(grp.get("keep", grp.get("count", 1)))),
+                                              None if not sh else int(sh["ff"])))
+            else:
+                raise NotImplementedError(f"layer {i}: mlp kind {mlp.get('kind')!r}")
+        return HybridConfig(name=str(cfg["architecture"]), vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers, eps=float(cfg["norm"]["eps"]),
+                            residual_mult=1.0, logit_softcap=0.0, norm_offset=0.0, shared_norm=True, branch_gates=True)
+
+
+_READERS = {"nufalorn": HybridConfig.nufalorn_from_json, "pokepel": HybridConfig.pokepel_from_json}
+
 
 class HybridModel:
     """Device weights + the step function.  dtype: torch.bfloat16 (16-bit weights and activations, fp32 accumulation and fp32 for everything
@@ -98,23 +154,46 @@ class HybridModel:
             if L.kind == "attention":
                 names = ["q", "o"] + (["k", "v"] if L.mixer.kv_from is None else [])
                 mixer = PagedChunkAttention(L.mixer, sub(p + "mix.", names), cfg.eps, page, self.device)
+            elif L.kind == "latent_attention":
+                mixer = LatentAttention(L.mixer, sub(p + "mix.", ["q", "dkv", "dkv.norm", "uk", "uv", "sink", "g", "o"]), cfg.eps, page, self.device)
+            elif L.kind == "retention":
+                mixer = Retention(L.mixer, sub(p + "mix.", ["q", "k", "v", "g", "o"]), cfg.eps, self.device)
             elif L.kind == "hgrn2":
                 mixer = GatedLinearRecurrence(L.mixer, sub(p + "mix.", ["q", "f", "f.b", "lower", "v", "norm", "o"]), cfg.eps)
             else:
                 mixer = GatedLinearRecurrence(L.mixer, sub(p + "mix.", ["q", "k", "v", "g", "a1", "a2", "a2.b", "norm", "o"]), cfg.eps)
             mlp = None
             if L.ff is not None:
-                mlp = GatedMLP(get(p + "mlp.gate"), get(p + "mlp.up"), get(p + "mlp.down"), L.mlp_act)
-            self.layers.append((L, mixer, mlp, get(p + "norm1"), get(p + "norm2") if mlp is not None else None))
-        self.has_state = any(L.kind != "attention" for L in cfg.layers)
+                gated = lambda q, act: GatedMLP(get(q + "gate"), get(q + "up"), get(q + "down"), act)
+                if L.mlp_kind == "gated":
+                    mlp = gated(p + "mlp.", L.mlp_act)
+                elif L.mlp_kind == "polynorm":
+                    mlp = PolyNormMLP(get(p + "mlp.up"), get(p + "mlp.down"), tensors[p + "mlp.act"], cfg.eps)
+                else:
+                    ex = [p + f"mlp.e{j}." for j in range(L.router.experts)]
+                    mlp = RoutedExperts(L.router, get(p + "mlp.router"), [get(q + "gate") for q in ex], [get(q + "up") for q in ex],
+                                        [get(q + "down") for q in ex], gated(p + "mlp.shared.", L.mlp_act) if L.shared_ff is not None else None, L.mlp_act)
+            gate_w = gate_b = None
+            if cfg.branch_gates:                       # both gates in one linear: columns [0, W) scale the mixer, [W, 2W) the MLP
+                names = ["rg1"] + (["rg2"] if mlp is not None else [])
+                gate_w = torch.cat([get(p + n) for n in names], 0).contiguous()
+                gate_b = torch.cat([get(p + n + ".b") for n in names], 0).contiguous()
+                if mlp is None:                        # the kernel reads two gates per row: keep the row stride at 2 W
+                    gate_w = torch.cat([gate_w, torch.zeros_like(gate_w)], 0).contiguous()
+                    gate_b = torch.cat([gate_b, torch.zeros_like(gate_b)], 0).contiguous()
+            n2 = get(p + "norm2") if mlp is not None and not cfg.shared_norm else None
+            self.layers.append((L, mixer, mlp, get(p + "norm1"), n2, gate_w, gate_b))
+        self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
 
     # ---- what an engine has to allocate
     def cache_layout(self):
-        """Per layer: ("kv", K page shape, V page shape) | ("kv_from", layer) | ("state", per-slot shape)."""
+        """Per layer: ("kv", K page shape, V page shape) | ("kv_from", layer) | ("latent", page shape) | ("state", per-slot shape)."""
         out = []
-        for L, mixer, _, _, _ in self.layers:
+        for L, mixer, *_ in self.layers:
             if L.kind == "attention":
                 out.append(("kv",) + mixer.cache_shapes() if mixer.owns_cache else ("kv_from", L.mixer.kv_from))
+            elif L.kind == "latent_attention":
+                out.append(("latent", mixer.cache_shape()))
             else:
                 out.append(("state", mixer.state_shape()))
         return out
@@ -128,6 +207,8 @@ class HybridModel:
                                torch.zeros(num_pages, *ent[2], dtype=self.dtype, device=self.device)))
             elif ent[0] == "kv_from":
                 caches.append(caches[ent[1]])
+            elif ent[0] == "latent":                   # one row per token serves as key and (its leading channels) as value
+                caches.append((torch.zeros(num_pages, *ent[1], dtype=self.dtype, device=self.device), None))
             else:
                 caches.append(torch.zeros(num_slots, *ent[1], dtype=torch.float32, device=self.device))
         return caches
@@ -138,18 +219,21 @@ class HybridModel:
         the residual stream after every layer (debugging / tests; costs one extra norm launch per layer)."""
         cfg = self.cfg
         x = hops.embed(batch.tokens, self.embed)
-        a = b = None
-        for (L, mixer, mlp, n1, n2), cache in zip(self.layers, caches):
-            h1, h2 = hops.residual_norm(x, a, b, cfg.residual_mult, n1, n2, cfg.eps, weight_offset=cfg.norm_offset)
+        a = b = g = None
+        for (L, mixer, mlp, n1, n2, gate_w, gate_b), cache in zip(self.layers, caches):
+            h1, h2 = hops.residual_norm(x, a, b, cfg.residual_mult, n1, n2, cfg.eps, weight_offset=cfg.norm_offset, gate=g)
             if collect is not None and a is not None:
                 collect.append(x.clone())
-            a = mixer.forward(h1, batch, *cache) if L.kind == "attention" else mixer.forward(h1, batch, cache)
+            if cfg.shared_norm:
+                h2 = h1
+            g = hops.dense_linear(h1, gate_w, gate_b, out_dtype=torch.float32) if gate_w is not None else None
+            a = mixer.forward(h1, batch, *cache) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache)
             b = mlp.forward(h2) if mlp is not None else None
         if collect is not None:
-            hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset)
+            hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, gate=g)
             collect.append(x.clone())
-            a = b = None
-        hf, _ = hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want)
+            a = b = g = None
+        hf, _ = hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, rows=batch.want, gate=g)
         return hops.dense_linear(hf, self.head, out_dtype=torch.float32, softcap=cfg.logit_softcap)
 
 

@@ -11,7 +11,7 @@ from . import _C
 
 ACT_NONE, ACT_RELU, ACT_SILU = 0, 1, 2
 ACTIVATIONS = {"none": ACT_NONE, "relu": ACT_RELU, "silu": ACT_SILU}
-SCAN_HGRN2, SCAN_GLA = 0, 1
+SCAN_HGRN2, SCAN_GLA, SCAN_FIXED = 0, 1, 2
 LAYOUTS = {"interleaved": 0, "halves": 1}
 
 
@@ -103,9 +103,11 @@ def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 
 def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.Tensor], mult: float, w1: torch.Tensor,
-                  w2: Optional[torch.Tensor], eps: float, *, weight_offset: float = 0.0, rows: Optional[torch.Tensor] = None):
+                  w2: Optional[torch.Tensor], eps: float, *, weight_offset: float = 0.0, rows: Optional[torch.Tensor] = None,
+                  gate: Optional[torch.Tensor] = None):
     """x <- x + mult * (a + b) on the fp32 stream (in place; skipped for absent branches, and x is only read when `rows` gathers), then
-    RMS norms of the new rows under w1 and w2 (stored weight + weight_offset).  -> (h1, h2) in the weights' dtype."""
+    RMS norms of the new rows under w1 and w2 (stored weight + weight_offset).  -> (h1, h2) in the weights' dtype.
+    gate: fp32 [T, >= 2 W] pre-activations; a is multiplied by sigmoid(gate[:, :W]) and b by sigmoid(gate[:, W:2W]) before they are added."""
     _dev(x, torch.float32, "residual_norm.x")
     W = x.shape[1]
     n = x.shape[0] if rows is None else rows.numel()
@@ -116,19 +118,26 @@ def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.
                 raise _C.Mi355Error(f"residual_norm.{nm}: {tuple(t.shape)} against the stream {tuple(x.shape)}")
     if rows is not None:
         _dev(rows, torch.int32, "residual_norm.rows")
+    ldg = 0
+    if gate is not None:
+        _dev(gate, torch.float32, "residual_norm.gate")
+        ldg = _rows(gate, "residual_norm.gate")
+        if gate.shape[0] != x.shape[0] or gate.shape[1] < 2 * W:
+            raise _C.Mi355Error(f"residual_norm.gate: {tuple(gate.shape)} for two gates of the stream {tuple(x.shape)}")
     if not x.is_contiguous() or w1.numel() != W or (w2 is not None and (w2.numel() != W or w2.dtype != w1.dtype)):
         raise _C.Mi355Error("residual_norm: stream must be contiguous and the weights [W] of one dtype")
     h1 = torch.empty(n, W, dtype=w1.dtype, device=x.device)
     h2 = torch.empty(n, W, dtype=w1.dtype, device=x.device) if w2 is not None else None
     if n:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_residual_norm(x.data_ptr(), _p(a), _p(b), float(mult), _p(rows), n, W, w1.data_ptr(), _p(w2),
-                                                               float(weight_offset), float(eps), h1.data_ptr(), _p(h2), act_code(w1.dtype),
-                                                               _stream()), "hy_residual_norm")
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_gated_residual_norm(x.data_ptr(), _p(a), _p(b), _p(gate), ldg, float(mult), _p(rows), n, W,
+                                                                     w1.data_ptr(), _p(w2), float(weight_offset), float(eps), h1.data_ptr(), _p(h2),
+                                                                     act_code(w1.dtype), _stream()), "hy_residual_norm")
     return h1, h2
 
 
-def attn_geometry(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages):
-    return (C.c_int32 * 10)(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages)
+def attn_geometry(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages, v_ld=0):
+    """v_ld: row stride of the value cache in elements (0: vdim; wider when the value rows are a leading part of wider cached rows)."""
+    return (C.c_int32 * 11)(heads, kv_heads, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages, v_ld)
 
 
 def attn_prep(qkv: torch.Tensor, koff: int, voff: int, geom, kfreq, vfreq, v_norm: bool, eps: float, pos, seq, block_table,
@@ -146,13 +155,23 @@ def attn_prep(qkv: torch.Tensor, koff: int, voff: int, geom, kfreq, vfreq, v_nor
                                                        _stream()), "hy_attn_prep")
 
 
-def attn_rows(q: torch.Tensor, scale: float, geom, chunk: int, sink: bool, vfreq, pos, seq, block_table, kcache, vcache, heads: int, vdim: int):
-    """Attention of every row over its sequence's pages -> [T, heads * vdim] in the cache dtype."""
+def _sink(sink: Optional[torch.Tensor], heads: int):
+    if sink is not None:
+        _dev(sink, torch.float32, "attention.sink")
+        if sink.numel() != heads or not sink.is_contiguous():
+            raise _C.Mi355Error(f"attention.sink: {tuple(sink.shape)} for {heads} heads")
+    return _p(sink)
+
+
+def attn_rows(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[torch.Tensor], vfreq, pos, seq, block_table, kcache, vcache,
+              heads: int, vdim: int):
+    """Attention of every row over its sequence's pages -> [T, heads * vdim] in the cache dtype.  sink: fp32 [heads] or None; exp(sink[h])
+    joins head h's softmax denominator."""
     _dev(q, torch.float32, "attn_rows.q")
     T = q.shape[0]
     out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_rows(q.data_ptr(), _rows(q, "attn_rows.q"), float(scale), geom, int(chunk), 1 if sink else 0, _p(vfreq),
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_rows(q.data_ptr(), _rows(q, "attn_rows.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
                                                            pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), T, kcache.data_ptr(), vcache.data_ptr(),
                                                            out.data_ptr(), act_code(kcache.dtype), _stream()), "hy_attn_rows")
     return out
@@ -163,7 +182,7 @@ def attn_tiles_supported(dtype: torch.dtype, dim: int, vdim: int, value_rot: boo
     return dtype == torch.bfloat16 and dim % 32 == 0 and dim <= 256 and vdim % 16 == 0 and vdim <= 256 and not (value_rot and v_layout and vdim % 32)
 
 
-def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: bool, vfreq, pos, seq, block_table, tile_row0, tile_n, kcache, vcache,
+def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[torch.Tensor], vfreq, pos, seq, block_table, tile_row0, tile_n, kcache, vcache,
                heads: int, vdim: int):
     """attn_rows for prompt portions on the matrix cores: tile t = rows tile_row0[t] .. + tile_n[t] - 1 (at most 16 consecutive rows of one
     sequence); every row of the batch must lie in exactly one tile."""
@@ -171,7 +190,7 @@ def attn_tiles(q: torch.Tensor, scale: float, geom, chunk: int, sink: bool, vfre
     T = q.shape[0]
     out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_tiles(q.data_ptr(), _rows(q, "attn_tiles.q"), float(scale), geom, int(chunk), 1 if sink else 0, _p(vfreq),
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_tiles(q.data_ptr(), _rows(q, "attn_tiles.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
                                                             pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), tile_row0.data_ptr(), tile_n.data_ptr(),
                                                             tile_row0.numel(), kcache.data_ptr(), vcache.data_ptr(), out.data_ptr(),
                                                             act_code(kcache.dtype), _stream()), "hy_attn_tiles")
@@ -193,13 +212,158 @@ def scan(mode: int, proj: torch.Tensor, qo: int, ko: int, vo: int, z: Optional[t
     return out
 
 
-def head_norm(o: torch.Tensor, heads: int, vdim: int, w: torch.Tensor, eps: float, gate: Optional[torch.Tensor] = None, goff: int = 0) -> torch.Tensor:
-    """Per-head RMS norm of o (fp32 [T, heads * vdim]) under the shared weight w [vdim], times silu(gate[:, goff:]) when a gate is given."""
+def head_norm(o: torch.Tensor, heads: int, vdim: int, w: Optional[torch.Tensor], eps: float, gate: Optional[torch.Tensor] = None, goff: int = 0,
+              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Per-head RMS norm of o (fp32 [T, heads * vdim]) under the shared weight w [vdim] (None: unit RMS only, output in `out_dtype`),
+    times silu(gate[:, goff:]) when a gate is given."""
     _dev(o, torch.float32, "head_norm.o")
     T = o.shape[0]
-    out = torch.empty(T, heads * vdim, dtype=w.dtype, device=o.device)
+    dt = w.dtype if w is not None else out_dtype
+    out = torch.empty(T, heads * vdim, dtype=dt, device=o.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_head_norm(o.data_ptr(), T, heads, vdim, w.data_ptr(), float(eps), _p(gate),
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_head_norm(o.data_ptr(), T, heads, vdim, _p(w), float(eps), _p(gate),
                                                            0 if gate is None else _rows(gate, "head_norm.gate"), goff, out.data_ptr(),
-                                                           act_code(w.dtype), _stream()), "hy_head_norm")
+                                                           act_code(dt), _stream()), "hy_head_norm")
+    return out
+
+
+def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: int = 0, offs: Optional[torch.Tensor] = None,
+                  gather: Optional[torch.Tensor] = None, rows: Optional[int] = None, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
+                  act: int = ACT_NONE, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One launch of G = w.shape[0] linears with the weights w [G, N, K].
+    Without offs every group takes all rows of x, reads its K inputs from column g * x_step and writes its outputs from column g * y_step
+    (per-head projections).  With offs (int32 [G + 1] on the device) the `rows` rows of the output are sorted by group, group g owns rows
+    offs[g] .. offs[g + 1] - 1, and sorted row r reads x[gather[r]] (x[r] without gather): the experts of a mixture."""
+    _dev(x, w.dtype, "dense_grouped.x"); _dev(w, w.dtype, "dense_grouped.w")
+    if w.dim() != 3 or not w.is_contiguous():
+        raise _C.Mi355Error(f"dense_grouped: weights {tuple(w.shape)} must be contiguous [G, N, K]")
+    G, N, K = w.shape
+    ldx = _rows(x, "dense_grouped.x")
+    M = x.shape[0] if rows is None else int(rows)
+    if gated and N % 64:
+        raise _C.Mi355Error(f"dense_grouped: a gated weight has whole groups of 64 rows, N={N}")
+    n_out = N // 2 if gated else N
+    od = torch.float32 if w.dtype == torch.float32 else (out_dtype or w.dtype)
+    width = y_step * (G - 1) + n_out if offs is None else n_out
+    if out is None:
+        out = torch.empty(M, width, dtype=od, device=x.device)
+    else:
+        _dev(out, od, "dense_grouped.out")
+        if out.shape[0] != M or out.shape[1] < width:
+            raise _C.Mi355Error(f"dense_grouped: out {tuple(out.shape)} for [{M}, {width}]")
+    if x.shape[1] < x_step * (G - 1) + K:
+        raise _C.Mi355Error(f"dense_grouped: x {tuple(x.shape)} for {G} groups of K={K} at step {x_step}")
+    for t, nm in ((offs, "offs"), (gather, "gather")):
+        if t is not None:
+            _dev(t, torch.int32, "dense_grouped." + nm)
+    if offs is not None and offs.numel() != G + 1:
+        raise _C.Mi355Error(f"dense_grouped: offs has {offs.numel()} entries for {G} groups")
+    if gather is not None and gather.numel() < M:
+        raise _C.Mi355Error(f"dense_grouped: gather has {gather.numel()} entries for {M} rows")
+    if M:
+        _C.check_hybrid(_C.hybrid_lib().mi355_dense_grouped(x.data_ptr(), ldx, M, w.data_ptr(), N, K, None, out.data_ptr(), _rows(out, "dense_grouped.out"),
+                                                            1 if od == torch.float32 else 0, 1 if gated else 0, act, act_code(w.dtype), G, x_step, y_step,
+                                                            _p(offs), _p(gather), _stream()), "dense_grouped")
+    return out
+
+
+def latent_geometry(heads, dim, rot_dim, rank, padded, rot_span, page, max_blocks, num_pages):
+    return (C.c_int32 * 9)(heads, dim, rot_dim, rank, padded, rot_span, page, max_blocks, num_pages)
+
+
+def latent_prep(proj: torch.Tensor, doff: int, geom, freq, mag: float, cw: torch.Tensor, eps: float, pos, seq, block_table, qn: torch.Tensor,
+                qabs: torch.Tensor, cache: torch.Tensor):
+    """Latent attention, before the scores: from the fp32 projections [T, ld] (query heads from column 0, down projection from column doff) write
+    the token's cached row [normed latent | turned shared key part | zeros], the un-rotated query parts (qn, activation dtype) and the turned
+    query parts + padding into columns rank.. of every head's absorbed query row (qabs fp32)."""
+    _dev(proj, torch.float32, "latent_prep.proj"); _dev(qabs, torch.float32, "latent_prep.qabs")
+    _dev(qn, cache.dtype, "latent_prep.qn"); _dev(cw, cache.dtype, "latent_prep.norm")
+    T = proj.shape[0]
+    H, dim, dr, R, dpad = geom[0], geom[1], geom[2], geom[3], geom[4]
+    if qn.shape != (T, H * dim) or qabs.shape != (T, H * dpad) or not qn.is_contiguous() or not qabs.is_contiguous() or cw.numel() != R:
+        raise _C.Mi355Error(f"latent_prep: qn {tuple(qn.shape)} qabs {tuple(qabs.shape)} norm {tuple(cw.shape)}")
+    if cache.dim() != 3 or cache.shape[1:] != (geom[6], dpad) or cache.shape[0] != geom[8] or not cache.is_contiguous():
+        raise _C.Mi355Error(f"latent_prep: cache {tuple(cache.shape)} against pages of {geom[6]} rows of {dpad}")
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_latent_prep(proj.data_ptr(), _rows(proj, "latent_prep.proj"), doff, geom, _p(freq), float(mag), cw.data_ptr(),
+                                                             float(eps), pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), T, qn.data_ptr(),
+                                                             qabs.data_ptr(), cache.data_ptr(), act_code(cache.dtype), _stream()), "hy_latent_prep")
+
+
+def rotary(buf: torch.Tensor, segments, rot_dims: int, layout: int, freq: torch.Tensor, mag: float, pos: torch.Tensor):
+    """Turn, in place, the first rot_dims channels of every head of up to two segments (column, heads, head size, scale) of the fp32 rows of buf
+    by position * freq (cos and sin times mag); a segment's heads are multiplied by its scale afterwards."""
+    _dev(buf, torch.float32, "rotary.buf")
+    segs = list(segments) + [(0, 0, 0, 1.0)] * (2 - len(segments))
+    if len(segs) != 2:
+        raise _C.Mi355Error("rotary: one or two segments")
+    if buf.shape[0]:
+        (o0, h0, d0, s0), (o1, h1, d1, s1) = segs
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_rotary(buf.data_ptr(), _rows(buf, "rotary.buf"), buf.shape[0], o0, h0, d0, float(s0), o1, h1, d1, float(s1),
+                                                        rot_dims, layout, _p(freq), float(mag), pos.data_ptr(), _stream()), "hy_rotary")
+
+
+def polynorm(z: torch.Tensor, coef, eps: float, dtype: torch.dtype) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e per row of the fp32 z, N = unit RMS over the row; coef = (a, b, c, e) -> `dtype`."""
+    _dev(z, torch.float32, "polynorm.z")
+    T, n = z.shape
+    out = torch.empty(T, n, dtype=dtype, device=z.device)
+    if T:
+        a, b, c, e = [float(v) for v in coef]
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_polynorm(z.data_ptr(), _rows(z, "polynorm.z"), T, n, a, b, c, e, float(eps), out.data_ptr(), n,
+                                                          act_code(dtype), _stream()), "hy_polynorm")
+    return out
+
+
+def gate_mul(o: torch.Tensor, gate: torch.Tensor, goff: int, dtype: torch.dtype) -> torch.Tensor:
+    """o * sigmoid(gate[:, goff : goff + n]) for fp32 o [T, n] -> `dtype`."""
+    _dev(o, torch.float32, "gate_mul.o"); _dev(gate, torch.float32, "gate_mul.gate")
+    if not o.is_contiguous():
+        raise _C.Mi355Error("gate_mul: o must be contiguous")
+    T, n = o.shape
+    out = torch.empty(T, n, dtype=dtype, device=o.device)
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_gate_mul(o.data_ptr(), T, n, gate.data_ptr(), _rows(gate, "gate_mul.gate"), goff, out.data_ptr(),
+                                                          act_code(dtype), _stream()), "hy_gate_mul")
+    return out
+
+
+def moe_route(z: torch.Tensor, groups: int, keep: int, top: int):
+    """Router logits fp32 [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]): softmax scores, only experts of the `keep` best of
+    `groups` runs of neighbouring experts (a run scores as its best member) are eligible, the `top` best eligible are chosen."""
+    _dev(z, torch.float32, "moe_route.z")
+    T, E = z.shape
+    ids = torch.empty(T, top, dtype=torch.int32, device=z.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route(z.data_ptr(), _rows(z, "moe_route.z"), T, E, groups, keep, top, ids.data_ptr(), wts.data_ptr(),
+                                                           _stream()), "hy_moe_route")
+    return ids, wts
+
+
+def moe_align(ids: torch.Tensor, experts: int):
+    """ids int32 [T, top] -> (offs int32 [E + 1], src_row int32 [T * top], place_of int32 [T * top]): the (token, choice) pairs sorted by
+    expert; sorted place p belongs to token src_row[p], pair i sits at place_of[i]."""
+    _dev(ids, torch.int32, "moe_align.ids")
+    T, top = ids.shape
+    offs = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
+    src = torch.empty(T * top, dtype=torch.int32, device=ids.device)
+    place = torch.empty(T * top, dtype=torch.int32, device=ids.device)
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_align(ids.data_ptr(), T * top, top, experts, offs.data_ptr(), src.data_ptr(), place.data_ptr(), _stream()),
+                        "hy_moe_align")
+    return offs, src, place
+
+
+def moe_combine(y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = sum_k wts[t, k] * y[place_of[t, k]] (+ extra[t]) -> fp32 [T, W]."""
+    _dev(y, torch.float32, "moe_combine.y"); _dev(wts, torch.float32, "moe_combine.wts")
+    T, top = wts.shape
+    W = y.shape[1]
+    if not y.is_contiguous() or y.shape[0] != T * top or (extra is not None and (extra.shape != (T, W) or extra.dtype != torch.float32 or not extra.is_contiguous())):
+        raise _C.Mi355Error(f"moe_combine: y {tuple(y.shape)} for {T} tokens x {top}")
+    out = torch.empty(T, W, dtype=torch.float32, device=y.device)
+    if T:
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_combine(y.data_ptr(), T, W, place_of.data_ptr(), wts.data_ptr(), top, _p(extra), out.data_ptr(), _stream()),
+                        "hy_moe_combine")
     return out

@@ -9,7 +9,15 @@
     HGRN2 parametrisation (a = f, k = 1 - f with a lower-bounded forget gate f, q = silu) or the gated-linear-attention one
     (a = sigmoid(low-rank z)^(1/tau), q scaled by dim^-1/2, output gate silu(g)); per-head RMS norm of o, then the output projection.
 
-Both take the normed activations of a ragged batch (``StepBatch``) and return the fp32 branch output [T, width]."""
+  * ``LatentAttention`` -- attention whose keys and values are linear images of ONE low-rank latent vector per token, plus a rotated key
+    part shared by all heads.  Only the normed latent and that key part are cached (one row per token for all heads); the key
+    up-projection is moved to the query side and the value up-projection behind the weighted sum, so the paged kernels see multi-query
+    attention over the cached rows.  Rotary with optional YaRN frequency scaling, a learned per-head softmax sink, a sigmoid output gate.
+  * ``Retention`` -- the same recurrence with one constant decay per head, rotated q and k, unit-RMS heads and a silu output gate.
+  * ``GatedMLP``, ``PolyNormMLP``, ``RoutedExperts`` -- feed-forward branches: gated dense, dense with the PolyNorm activation, and a
+    mixture of gated experts (softmax router, group-limited top-k, optional shared expert) over one grouped linear per projection.
+
+All take the normed activations of a ragged batch (``StepBatch``) and return the fp32 branch output [T, width]."""
 import math
 from dataclasses import dataclass
 from typing import Dict, Optional
@@ -20,10 +28,29 @@ from . import hybrid_ops as hops
 
 
 @dataclass
+class RotaryScaling:
+    """YaRN: pairs that turn fewer than `slow` times over `original` positions are slowed by `factor`, pairs that turn more than `fast`
+    times keep their step, with a linear ramp over the pair index between; cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass
 class RotarySpec:
     dims: int
     base: float
     layout: str = "interleaved"          # "interleaved": pairs (2i, 2i+1); "halves": (i, i + dims / 2)
+    scaling: Optional[RotaryScaling] = None
+
+    @staticmethod
+    def from_json(rot: Optional[dict], layout: str) -> Optional["RotarySpec"]:
+        if not rot or not int(rot.get("dims", 0)):
+            return None
+        sc = rot.get("scaling")
+        return RotarySpec(int(rot["dims"]), float(rot["base"]), layout,
+                          RotaryScaling(float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"])) if sc else None)
 
 
 @dataclass
@@ -35,7 +62,7 @@ class AttentionSpec:
     scale: float
     rot: Optional[RotarySpec] = None
     chunk: int = 0                       # 0: every earlier position is visible
-    sink: bool = False
+    sink: bool = False                   # exp(0) joins the softmax denominator
     value_norm: bool = False
     value_rot: bool = False
     value_layout: str = "interleaved"
@@ -69,6 +96,20 @@ class StepBatch:
     host: Optional[torch.Tensor] = None        # the pinned buffer all index fields were uploaded from (one copy per step)
 
 
+def rotary_table(rot: RotarySpec, device):
+    """(fp32 angular steps [dims / 2] on the device, magnitude of cos and sin) of a rotary description; evaluated in float64, rounded once."""
+    i = torch.arange(rot.dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(rot.base), dtype=torch.float64), -2.0 * i / rot.dims)
+    mag, sc = 1.0, rot.scaling
+    if sc is not None:
+        at = lambda turns: rot.dims * math.log(sc.original / (2.0 * math.pi * turns)) / (2.0 * math.log(rot.base))
+        lo, hi = max(math.floor(at(sc.fast)), 0), min(math.ceil(at(sc.slow)), rot.dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / sc.factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(sc.factor) + 1.0
+    return f.to(torch.float32).to(device), mag
+
+
 def rotary_steps(n_pairs: int, span: int, base: float, device) -> torch.Tensor:
     """fp32 angular step of pair i: base^(-2 i / span), evaluated in float64 and rounded once."""
     i = torch.arange(n_pairs, dtype=torch.float64)
@@ -91,6 +132,7 @@ class PagedChunkAttention:
         self.vfreq = rotary_steps(s.vdim // 2, s.vdim, rot.base, device) if s.value_rot and rot else None
         self._geom = None
         self.use_tiles = True
+        self.sink = torch.zeros(s.heads, dtype=torch.float32, device=device) if s.sink else None
 
     def cache_shapes(self):
         """(K page tensor shape, V page tensor shape) without the leading page count."""
@@ -118,10 +160,10 @@ class PagedChunkAttention:
         # prompt portions (tiles mostly full) go to the matrix-core kernel, decode rows to the one that spreads a row's keys over four waves
         if (self.use_tiles and batch.tile_row0 is not None and batch.tile_row0.numel() * 4 <= T
                 and hops.attn_tiles_supported(kcache.dtype, s.dim, s.vdim, self.vfreq is not None, hops.LAYOUTS[s.value_layout])):
-            o = hops.attn_tiles(qkv, s.scale, geom, s.chunk, s.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n,
+            o = hops.attn_tiles(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n,
                                 kcache, vcache, s.heads, s.vdim)
         else:
-            o = hops.attn_rows(qkv, s.scale, geom, s.chunk, s.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim)
+            o = hops.attn_rows(qkv, s.scale, geom, s.chunk, self.sink, self.vfreq, batch.pos, batch.seq, batch.block_table, kcache, vcache, s.heads, s.vdim)
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
 
@@ -160,6 +202,177 @@ class GatedLinearRecurrence:
                       batch.row_start, batch.slot, batch.first_pos, state, self.act)
         o = hops.head_norm(o, s.heads, s.vdim, self.norm, self.eps, proj if self.go is not None else None, self.go or 0)
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
+
+
+@dataclass
+class LatentAttentionSpec:
+    heads: int
+    dim: int                             # un-rotated query / key channels per head
+    rot_dim: int                         # rotated channels per head (the key's are shared by all heads)
+    vdim: int
+    kv_rank: int                         # size of the cached latent
+    scale: float
+    rot: Optional[RotarySpec] = None     # turns the first rot.dims of the rot_dim channels
+    sink: bool = True                    # learned per-head sink logit in the softmax denominator
+    out_gate: bool = True                # heads multiplied by sigmoid(W_g h) before the output projection
+
+
+class LatentAttention:
+    """weights: q [H (dim + rot_dim), W], dkv [kv_rank + rot_dim, W], dkv.norm [kv_rank], uk [H dim, kv_rank], uv [H vdim, kv_rank], sink [H],
+    g [H vdim, W], o [W, H vdim].  Cached per token: [normed latent | turned shared key part | zeros] in `padded` channels (a multiple of 32,
+    so that the matrix-core attention takes the rows); the values are the first kv_rank channels of the same row."""
+
+    def __init__(self, spec: LatentAttentionSpec, weights: Dict[str, torch.Tensor], eps: float, page: int, device):
+        s = self.spec = spec
+        self.eps, self.page = eps, page
+        H, d, dr, R = s.heads, s.dim, s.rot_dim, s.kv_rank
+        self.padded = -(-(R + dr) // 32) * 32
+        if s.rot is not None and (s.rot.dims > dr or s.rot.layout != "interleaved"):
+            raise ValueError(f"latent attention: rotary span {s.rot.dims} of {dr} channels ({s.rot.layout})")
+        parts = [weights["q"], weights["dkv"]] + ([weights["g"]] if s.out_gate else [])
+        self.w_in = torch.cat(parts, 0).contiguous()
+        self.doff, self.goff = H * (d + dr), H * (d + dr) + R + dr
+        self.c_norm = weights["dkv.norm"].contiguous()
+        # key up-projection on the query side: per head [kv_rank, dim] (q_abs = W_uk,h^T q_h); value up-projection per head [vdim, kv_rank]
+        self.w_uk_t = weights["uk"].view(H, d, R).transpose(1, 2).contiguous()
+        self.w_uv = weights["uv"].view(H, s.vdim, R).contiguous()
+        self.w_o = weights["o"].contiguous()
+        self.sink = weights["sink"].to(torch.float32).contiguous() if s.sink else None
+        self.freq, self.mag = rotary_table(s.rot, device) if s.rot is not None else (None, 1.0)
+        self.act = self.w_o.dtype
+        self._geom = None
+        self.use_tiles = True
+
+    def cache_shape(self):
+        return (self.page, self.padded)
+
+    def geometry(self, max_blocks: int, num_pages: int):
+        s = self.spec
+        key = (max_blocks, num_pages)
+        if self._geom is None or self._geom[0] != key:
+            self._geom = (key, hops.attn_geometry(s.heads, 1, self.padded, s.kv_rank, 0, 0, 0, self.page, max_blocks, num_pages, v_ld=self.padded),
+                          hops.latent_geometry(s.heads, s.dim, s.rot_dim, s.kv_rank, self.padded, s.rot.dims if s.rot else 0, self.page, max_blocks,
+                                               num_pages))
+        return self._geom[1], self._geom[2]
+
+    def forward(self, h: torch.Tensor, batch: StepBatch, cache: torch.Tensor, _values=None) -> torch.Tensor:
+        s = self.spec
+        H, R = s.heads, s.kv_rank
+        ageom, lgeom = self.geometry(batch.block_table.shape[1], cache.shape[0])
+        T = h.shape[0]
+        proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        qn = torch.empty(T, H * s.dim, dtype=self.act, device=h.device)
+        qabs = torch.empty(T, H * self.padded, dtype=torch.float32, device=h.device)
+        hops.latent_prep(proj, self.doff, lgeom, self.freq, self.mag, self.c_norm, self.eps, batch.pos, batch.seq, batch.block_table, qn, qabs, cache)
+        hops.dense_grouped(qn, self.w_uk_t, x_step=s.dim, y_step=self.padded, out_dtype=torch.float32, out=qabs)
+        kc = cache.view(cache.shape[0], 1, self.page, self.padded)
+        if (self.use_tiles and batch.tile_row0 is not None and batch.tile_row0.numel() * 4 <= T
+                and hops.attn_tiles_supported(cache.dtype, self.padded, R, False, 0)):
+            ol = hops.attn_tiles(qabs, s.scale, ageom, 0, self.sink, None, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n, kc, kc, H, R)
+        else:
+            ol = hops.attn_rows(qabs, s.scale, ageom, 0, self.sink, None, batch.pos, batch.seq, batch.block_table, kc, kc, H, R)
+        o = hops.dense_grouped(ol, self.w_uv, x_step=R, y_step=s.vdim, out_dtype=torch.float32)
+        o = hops.gate_mul(o, proj, self.goff, self.act) if s.out_gate else o.to(self.act)
+        return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
+
+
+@dataclass
+class RetentionSpec:
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple                         # one constant decay per head
+    rot: Optional[RotarySpec] = None
+
+
+class Retention:
+    """weights: q, k [H dim, W], v, g [H vdim, W], o [W, H vdim].  S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with q and k turned by the
+    position and k multiplied by dim^-1/2 after the turn; every head's o is brought to unit RMS, the heads are multiplied by silu(W_g h)."""
+
+    def __init__(self, spec: RetentionSpec, weights: Dict[str, torch.Tensor], eps: float, device):
+        s = self.spec = spec
+        self.eps = eps
+        if len(s.decay) != s.heads:
+            raise ValueError(f"retention: {len(s.decay)} decays for {s.heads} heads")
+        hd = s.heads * s.dim
+        self.w_in = torch.cat([weights["q"], weights["k"], weights["v"], weights["g"]], 0).contiguous()
+        self.qo, self.ko, self.vo, self.go = 0, hd, 2 * hd, 2 * hd + s.heads * s.vdim
+        self.decay = torch.tensor([float(a) for a in s.decay], dtype=torch.float32, device=device)
+        self.w_o = weights["o"].contiguous()
+        self.act = self.w_o.dtype
+        self.freq, self.mag = rotary_table(s.rot, device) if s.rot is not None else (None, 1.0)
+
+    def state_shape(self):
+        s = self.spec
+        return (s.heads, s.dim, s.vdim)
+
+    def forward(self, h: torch.Tensor, batch: StepBatch, state: torch.Tensor) -> torch.Tensor:
+        s = self.spec
+        proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        rot = s.rot
+        hops.rotary(proj, [(self.qo, s.heads, s.dim, 1.0), (self.ko, s.heads, s.dim, 1.0 / math.sqrt(s.dim))], rot.dims if rot else 0,
+                    hops.LAYOUTS[rot.layout] if rot else 0, self.freq, self.mag, batch.pos)
+        o = hops.scan(hops.SCAN_FIXED, proj, self.qo, self.ko, self.vo, None, self.decay, None, 1.0, 1.0, s.heads, s.dim, s.vdim,
+                      batch.row_start, batch.slot, batch.first_pos, state, self.act)
+        o = hops.head_norm(o, s.heads, s.vdim, None, self.eps, proj, self.go, out_dtype=self.act)
+        return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
+
+
+class PolyNormMLP:
+    """down(a N(z) + b N(z^2) + c N(z^3) + e), z = up h, N = unit RMS over a token's hidden channels; coef = the four numbers (a, b, c, e)."""
+
+    def __init__(self, up: torch.Tensor, down: torch.Tensor, coef: torch.Tensor, eps: float):
+        self.w_up, self.w_down = up.contiguous(), down.contiguous()
+        self.coef = tuple(float(v) for v in coef.detach().to("cpu", torch.float32).flatten())
+        if len(self.coef) != 4:
+            raise ValueError(f"PolyNorm takes four coefficients, got {len(self.coef)}")
+        self.eps = eps
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        z = hops.dense_linear(h, self.w_up, out_dtype=torch.float32)
+        return hops.dense_linear(hops.polynorm(z, self.coef, self.eps, self.w_down.dtype), self.w_down, out_dtype=torch.float32)
+
+
+@dataclass
+class RouterSpec:
+    experts: int
+    top: int
+    groups: int = 1                      # experts form `groups` runs of neighbours ...
+    keep: int = 1                        # ... and only those of the `keep` best runs can be chosen
+
+
+class RoutedExperts:
+    """Mixture of gated experts down_e(act(gate_e h) * up_e h): fp32 softmax router, group-limited top-k, the chosen experts' outputs weighted
+    by their softmax scores (not renormalised), plus an optional shared expert that every token runs.  The (token, choice) pairs are sorted
+    by expert on the device and each projection of all experts is one grouped linear; nothing returns to the host."""
+
+    def __init__(self, router: RouterSpec, w_router: torch.Tensor, gates, ups, downs, shared: Optional["GatedMLP"] = None, act: str = "silu"):
+        r = self.router = router
+        if len(gates) != r.experts or w_router.shape[0] != r.experts:
+            raise ValueError(f"experts: router of {w_router.shape[0]}, {len(gates)} experts, config says {r.experts}")
+        if r.experts % r.groups or not 1 <= r.keep <= r.groups or not 1 <= r.top <= (r.experts // r.groups) * r.keep:
+            raise ValueError(f"experts: {r.experts} experts in {r.groups} groups, keep {r.keep}, top {r.top}")
+        self.w_router = w_router.contiguous()
+        ff, K = gates[0].shape
+        pad = (-ff) % 32
+        gu, dn = [], []
+        for g, u, d in zip(gates, ups, downs):
+            if pad:
+                z = torch.zeros(pad, K, dtype=g.dtype, device=g.device)
+                g, u = torch.cat([g, z]), torch.cat([u, z])
+                d = torch.cat([d, torch.zeros(d.shape[0], pad, dtype=d.dtype, device=d.device)], 1)
+            gu.append(hops.group_gate_up(g, u)); dn.append(d)
+        self.w_gate_up, self.w_down = torch.stack(gu).contiguous(), torch.stack(dn).contiguous()
+        self.shared, self.act = shared, hops.ACTIVATIONS[act]
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        r = self.router
+        ids, wts = hops.moe_route(hops.dense_linear(h, self.w_router, out_dtype=torch.float32), r.groups, r.keep, r.top)
+        offs, src, place = hops.moe_align(ids, r.experts)
+        n = ids.numel()
+        a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, rows=n, gated=True, act=self.act)
+        y = hops.dense_grouped(a, self.w_down, offs=offs, rows=n, out_dtype=torch.float32)
+        return hops.moe_combine(y, place, wts, self.shared.forward(h) if self.shared is not None else None)
 
 
 class GatedMLP:
