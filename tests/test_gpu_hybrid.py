@@ -389,7 +389,7 @@ def test_matrix_core_attention_for_portions_equals_row_kernel(dim, vdim, heads, 
     geom = hops.attn_geometry(heads, kv_heads, dim, vdim, dim, 0, hops.LAYOUTS[layout], page, width, num_pages)
     vf = rotary_steps(vdim // 2, vdim, 1e4, DEV)
     assert hops.attn_tiles_supported(torch.bfloat16, dim, vdim, True, hops.LAYOUTS[layout])
-    for sink, vfreq in ((True, vf), (False, None)):
+    for sink, vfreq in ((torch.zeros(heads, device=DEV), vf), (None, None)):
         a = hops.attn_rows(q, dim ** -0.5, geom, chunk, sink, vfreq, i32(pos), i32(seq), tables.to(DEV), kc, vc, heads, vdim)
         b = hops.attn_tiles(q, dim ** -0.5, geom, chunk, sink, vfreq, i32(pos), i32(seq), tables.to(DEV), i32(t0), i32(tn), kc, vc, heads, vdim)
         err = (a.float() - b.float()).abs()
