@@ -60,10 +60,11 @@ def latent_attention(h, wts, pre, mx, eps):
     H, d, dr, dv, R = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"], mx["kv_rank"]
     pos = torch.arange(T)
     q = (h @ wts[pre + "q"].T).view(T, H, d + dr)
-    q_plain, q_rot = q[..., :d], rotate(q[..., d:], pos, mx["rot"], "interleaved")
+    rot = mx.get("rot") or {"dims": 0}
+    q_plain, q_rot = q[..., :d], rotate(q[..., d:], pos, rot, "interleaved")
     down = h @ wts[pre + "dkv"].T
     c = rms_unit(down[:, :R], eps) * wts[pre + "dkv.norm"]
-    k_rot = rotate(down[:, None, R:], pos, mx["rot"], "interleaved")[:, 0]           # [T, dr], one for all heads
+    k_rot = rotate(down[:, None, R:], pos, rot, "interleaved")[:, 0]           # [T, dr], one for all heads
     k_plain = (c @ wts[pre + "uk"].T).view(T, H, d)
     v = (c @ wts[pre + "uv"].T).view(T, H, dv)
     out = torch.zeros(T, H, dv, dtype=h.dtype)
@@ -84,8 +85,9 @@ def retention(h, wts, pre, mx, eps):
     T = h.shape[0]
     H, d, dv = mx["heads"], mx["dim"], mx["vdim"]
     pos = torch.arange(T)
-    q = rotate((h @ wts[pre + "q"].T).view(T, H, d), pos, mx["rot"], "halves")
-    k = rotate((h @ wts[pre + "k"].T).view(T, H, d), pos, mx["rot"], "halves") * d ** -0.5
+    rot = mx.get("rot") or {"dims": 0}
+    q = rotate((h @ wts[pre + "q"].T).view(T, H, d), pos, rot, "halves")
+    k = rotate((h @ wts[pre + "k"].T).view(T, H, d), pos, rot, "halves") * d ** -0.5
     v = (h @ wts[pre + "v"].T).view(T, H, dv)
     o = torch.zeros(T, H, dv, dtype=h.dtype)
     for hh in range(H):
