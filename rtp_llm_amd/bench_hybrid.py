@@ -2,7 +2,12 @@
 the Qwen2 / Llama engine at equal width, depth, head geometry, FFN width and vocabulary (bf16, 16-bit weights), and the kernels of both
 against their rooflines (HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s, fp32 vector FMA 157 TFLOP/s).
 
-Output: one JSON line {"hybrid_bench": {size: {"hybrid": {...}, "qwen2": {...}, "kernels": [...]}}}."""
+`--hybrid-design pokepel` measures the Pokepel member (latent attention, retention, PolyNorm MLP, routed experts) beside the family's
+Nufalorn member at equal width, depth, heads, FFN width (active per token) and vocabulary, and Pokepel's kernels beside the like
+Nufalorn kernels against their rooflines.
+
+Output: one JSON line {"hybrid_bench": {size: {"hybrid": {...}, "qwen2": {...}, "kernels": [...]}}} (with --hybrid-design pokepel:
+{"pokepel": {...}, "nufalorn": {...}, "kernels": [...]})."""
 import json
 import math
 import sys
@@ -73,6 +78,59 @@ def hybrid_weights(cfg, dev, seed=0):
     return w
 
 
+POKEPEL_PATTERN = ["retention", "latent", "latent", "retention", "latent", "latent", "retention", "latent"]
+
+
+def pokepel_config(s, experts=16, top=4, groups=4, keep=2):
+    """Width, depth, heads and vocabulary of `s`; latent attention with a 192-channel latent + 64 rotated channels (one 256-channel cached row
+    per token), retention with the recurrent sizes of the GLA layers; the first layer has a PolyNorm MLP of the full FFN width, the others
+    `experts` experts of a quarter of it (`top` of them + one shared expert per token: 1.25 x the dense FFN's work)."""
+    layers, hd = [], s["hd"]
+    for i in range(s["layers"]):
+        kind = POKEPEL_PATTERN[i % len(POKEPEL_PATTERN)]
+        fe = s["ff"] // 4 // 32 * 32
+        mlp = {"kind": "dense", "ff": s["ff"]} if i == 0 else {"kind": "moe", "expert": {"ff": fe}, "shared": {"ff": fe},
+                                                               "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep}}}
+        if kind == "latent":
+            mx = {"heads": s["heads"], "dim": hd, "rot_dim": hd // 2, "vdim": hd, "kv_rank": 3 * hd // 2, "scale": (hd + hd // 2) ** -0.5,
+                  "rot": {"base": 1e6, "dims": hd // 2, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+            layers.append({"type": "latent_attention", "mixer": mx, "mlp": mlp})
+        else:
+            mx = {"heads": s["heads"], "dim": hd // 2, "vdim": hd, "decay": [1.0 - 2.0 ** -(5 + h % 8) for h in range(s["heads"])], "rot": {"base": 1e6, "dims": hd // 2}}
+            layers.append({"type": "retention", "mixer": mx, "mlp": mlp})
+    return {"architecture": "Pokepel", "layers": layers, "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}}
+
+
+def pokepel_weights(cfg, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    W = cfg["width"]
+    lin = lambda o, i: (torch.randn(o, i, device=dev, generator=g) * i ** -0.5).bfloat16()
+    vec = lambda n, k=0.1, off=0.0: (torch.randn(n, device=dev, generator=g) * k + off).bfloat16()
+    w = {"embed": (torch.randn(cfg["vocab"], W, device=dev, generator=g)).bfloat16(), "head": lin(cfg["vocab"], W), "final.norm": vec(W, 0.1, 1.0)}
+    for i, L in enumerate(cfg["layers"]):
+        p, mx, mlp = f"l{i}.", L["mixer"], L["mlp"]
+        H, d, dv = mx["heads"], mx["dim"], mx["vdim"]
+        w[p + "norm1"] = vec(W, 0.1, 1.0)
+        if L["type"] == "latent_attention":
+            dr, R = mx["rot_dim"], mx["kv_rank"]
+            for n, (o, k) in {"q": (H * (d + dr), W), "dkv": (R + dr, W), "uk": (H * d, R), "uv": (H * dv, R), "g": (H * dv, W), "o": (W, H * dv)}.items():
+                w[p + "mix." + n] = lin(o, k)
+            w[p + "mix.dkv.norm"], w[p + "mix.sink"] = vec(R, 0.1, 1.0), vec(H, 1.0)
+        else:
+            for n, (o, k) in {"q": (H * d, W), "k": (H * d, W), "v": (H * dv, W), "g": (H * dv, W), "o": (W, H * dv)}.items():
+                w[p + "mix." + n] = lin(o, k)
+        for n in ("rg1", "rg2"):
+            w[p + n], w[p + n + ".b"] = lin(W, W), vec(W, 0.5)
+        if mlp["kind"] == "dense":
+            w[p + "mlp.up"], w[p + "mlp.down"], w[p + "mlp.act"] = lin(mlp["ff"], W), lin(W, mlp["ff"]), torch.tensor([0.6, 0.3, 0.1, 0.0]).bfloat16()
+        else:
+            w[p + "mlp.router"] = lin(mlp["router"]["experts"], W)
+            for n in [f"e{j}" for j in range(mlp["router"]["experts"])] + ["shared"]:
+                f = mlp["expert"]["ff"]
+                w[p + f"mlp.{n}.gate"], w[p + f"mlp.{n}.up"], w[p + f"mlp.{n}.down"] = lin(f, W), lin(f, W), lin(W, f)
+    return w
+
+
 def timed(fn, reps=5, warm=2, graph=False):
     """Seconds per call.  graph: the calls are captured into one HIP graph and the replay is timed, so the figure is the kernels' own
     time and not the host's launch path (what a graph-replayed step pays)."""
@@ -104,11 +162,11 @@ def timed(fn, reps=5, warm=2, graph=False):
     return e0.elapsed_time(e1) / reps * 1e-3
 
 
-def bench_hybrid_engine(s, dev, prompt, batch, steps):
+def bench_hybrid_engine(s, dev, prompt, batch, steps, design="nufalorn"):
     from .hybrid import HybridConfig, HybridModel
     from .scheduler import ServingEngine
-    cfg = hybrid_config(s)
-    model = HybridModel(HybridConfig.from_json(cfg), hybrid_weights(cfg, dev), torch.bfloat16, dev)
+    cfg = pokepel_config(s) if design == "pokepel" else hybrid_config(s)
+    model = HybridModel(HybridConfig.from_json(cfg), (pokepel_weights if design == "pokepel" else hybrid_weights)(cfg, dev), torch.bfloat16, dev)
     eng = ServingEngine(model, max_tokens=batch * (prompt + 8 * (steps + 3) + 128), max_seqs=batch, max_step_tokens=1 << 20)
     g = torch.Generator().manual_seed(1)
     toks = lambda n: torch.randint(0, s["vocab"], (n,), generator=g).tolist()
@@ -208,18 +266,19 @@ def kernel_table(s, dev, prompt):
     kc, vc = bf(nblk, G, page, hd), bf(nblk, G, page, hd)
     bt = torch.arange(nblk, dtype=torch.int32, device=dev).reshape(1, nblk)
     vf = torch.ones(hd // 2, device=dev) * 1e-3
+    sink0 = torch.zeros(H, device=dev)
     for T_, name in ((prompt, "prefill"), (1, "decode")):
         pos = (torch.arange(T_, dtype=torch.int32, device=dev) if T_ > 1 else torch.tensor([prompt - 1], dtype=torch.int32, device=dev))
         seq = torch.zeros(T_, dtype=torch.int32, device=dev)
         q = torch.randn(T_, H * hd, device=dev, generator=g)
-        t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, chunk, True, vf, pos, seq, bt, kc, vc, H, hd))
+        t = timed_k(lambda: hops.attn_rows(q, hd ** -0.5, geom, chunk, sink0, vf, pos, seq, bt, kc, vc, H, hd))
         keys = float(sum(min(int(p) % chunk + 1, chunk) for p in pos.tolist()))
         add("hybrid", f"attn_rows {name} (chunk {chunk})", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t,
             min(prompt, chunk if T_ == 1 else prompt) * G * hd * 2 * 2 + T_ * H * hd * 6, 4.0 * keys * H * hd, MFMA_BF16)
         if T_ > 1:
             t0 = torch.arange(0, T_, 16, dtype=torch.int32, device=dev)
             tn = torch.full_like(t0, 16)
-            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, chunk, True, vf, pos, seq, bt, t0, tn, kc, vc, H, hd))
+            t = timed_k(lambda: hops.attn_tiles(q, hd ** -0.5, geom, chunk, sink0, vf, pos, seq, bt, t0, tn, kc, vc, H, hd))
             add("hybrid", f"attn_tiles {name} (chunk {chunk}, MFMA)", f"T={T_} H={H} G={G} hd={hd} ctx={prompt}", t,
                 prompt * G * hd * 2 * 2 + T_ * H * hd * 6, 4.0 * keys * H * hd, MFMA_BF16)
         kvb = torch.randn(nblk, 2, G, page, hd, device=dev, generator=g).bfloat16()
@@ -252,12 +311,171 @@ def kernel_table(s, dev, prompt):
     return rows
 
 
+def kernel_table_pokepel(s, dev, prompt):
+    """Pokepel's kernels at this size beside the like kernels of the Nufalorn member, against max(bytes / HBM, flops / peak of the unit)."""
+    from . import hybrid_ops as hops
+    rows = []
+    timed_k = lambda fn: timed(fn, reps=10, warm=2, graph=True)
+    g = torch.Generator(device=dev).manual_seed(3)
+    bf = lambda *sh: torch.randn(*sh, device=dev, generator=g).bfloat16()
+    f32 = lambda *sh: torch.randn(*sh, device=dev, generator=g)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    W, H, G, hd, ff = s["width"], s["heads"], s["kv"], s["hd"], s["ff"]
+    cfg = pokepel_config(s)
+    lat = next(L["mixer"] for L in cfg["layers"] if L["type"] == "latent_attention")
+    moe = next(L["mlp"] for L in cfg["layers"] if L["mlp"]["kind"] == "moe")
+    R, dr, fe, E, top = lat["kv_rank"], lat["rot_dim"], moe["expert"]["ff"], moe["router"]["experts"], moe["router"]["top"]
+    dpad = -(-(R + dr) // 32) * 32
+
+    def add(family, name, shape, t, nbytes, flops, peak):
+        roof = max(nbytes / HBM, flops / peak)
+        rows.append({"family": family, "kernel": name, "shape": shape, "us": round(t * 1e6, 1), "roofline_us": round(roof * 1e6, 2),
+                     "x_roofline": round(t / roof, 1)})
+
+    page = 64
+    nblk = (prompt + page - 1) // page + 1
+    bt = torch.arange(nblk, dtype=torch.int32, device=dev).reshape(1, nblk)
+    sink = f32(H)
+    # attention: one cached row of dpad channels per token for all heads (values = its first R channels) against grouped-query pages
+    geom = hops.attn_geometry(H, 1, dpad, R, 0, 0, 0, page, nblk, nblk, v_ld=dpad)
+    ngeom = hops.attn_geometry(H, G, hd, hd, hd, 0, 0, page, nblk, nblk)
+    kc = bf(nblk, 1, page, dpad)
+    nk, nv = bf(nblk, G, page, hd), bf(nblk, G, page, hd)
+    vf = torch.ones(hd // 2, device=dev) * 1e-3
+    for T_, name in ((prompt, "prefill"), (1, "decode")):
+        pos = torch.arange(T_, dtype=torch.int32, device=dev) if T_ > 1 else i32([prompt - 1])
+        seq = torch.zeros(T_, dtype=torch.int32, device=dev)
+        q, nq = f32(T_, H * dpad), f32(T_, H * hd)
+        keys = float(sum(int(p) + 1 for p in pos.tolist()))
+        ctx = prompt
+        if T_ > 1:
+            t0 = torch.arange(0, T_, 16, dtype=torch.int32, device=dev)
+            tn = torch.full_like(t0, 16)
+            t = timed_k(lambda: hops.attn_tiles(q, 0.07, geom, 0, sink, None, pos, seq, bt, t0, tn, kc, kc, H, R))
+            add("pokepel", "attn_tiles latent prefill (causal, MFMA)", f"T={T_} H={H} row={dpad} rank={R} ctx={ctx}", t, ctx * dpad * 2 + T_ * H * (dpad * 4 + R * 2),
+                2.0 * keys * H * (dpad + R), MFMA_BF16)
+            t = timed_k(lambda: hops.attn_tiles(nq, hd ** -0.5, ngeom, 0, sink, vf, pos, seq, bt, t0, tn, nk, nv, H, hd))
+            add("nufalorn", "attn_tiles prefill (causal, MFMA)", f"T={T_} H={H} G={G} hd={hd} ctx={ctx}", t, ctx * G * hd * 2 * 2 + T_ * H * hd * 6, 4.0 * keys * H * hd, MFMA_BF16)
+        else:
+            t = timed_k(lambda: hops.attn_rows(q, 0.07, geom, 0, sink, None, pos, seq, bt, kc, kc, H, R))
+            add("pokepel", "attn_rows latent decode", f"T=1 H={H} row={dpad} rank={R} ctx={ctx}", t, ctx * dpad * 2, 2.0 * keys * H * (dpad + R), MFMA_BF16)
+            t = timed_k(lambda: hops.attn_rows(nq, hd ** -0.5, ngeom, 0, sink, vf, pos, seq, bt, nk, nv, H, hd))
+            add("nufalorn", "attn_rows decode", f"T=1 H={H} G={G} hd={hd} ctx={ctx}", t, ctx * G * hd * 2 * 2, 4.0 * keys * H * hd, MFMA_BF16)
+    # before the scores: norm + turn + page write + query split, against turn + value norm + page write
+    lgeom = hops.latent_geometry(H, hd, dr, R, dpad, dr, page, nblk, nblk)
+    freq = torch.ones(dr // 2, device=dev) * 1e-3
+    for T_ in (prompt, 8):
+        pos, seq = torch.arange(T_, dtype=torch.int32, device=dev), torch.zeros(T_, dtype=torch.int32, device=dev)
+        proj, qn, qabs, cw = f32(T_, H * (hd + dr) + R + dr), bf(T_, H * hd), f32(T_, H * dpad), bf(R)
+        t = timed_k(lambda: hops.latent_prep(proj, H * (hd + dr), lgeom, freq, 1.2, cw, 1e-6, pos, seq, bt, qn, qabs, kc.view(nblk, page, dpad)))
+        add("pokepel", "latent_prep", f"T={T_} H={H}", t, T_ * (H * (hd + dr) * 4 + H * hd * 2 + H * (dpad - R) * 4 + dpad * 2), 0, VALU_F32)
+        qkv = f32(T_, (H + 2 * G) * hd)
+        t = timed_k(lambda: hops.attn_prep(qkv, H * hd, (H + G) * hd, ngeom, freq.repeat(2)[: hd // 2], vf, True, 1e-5, pos, seq, bt, nk, nv))
+        add("nufalorn", "attn_prep", f"T={T_} H={H} G={G}", t, T_ * ((H + 2 * G) * hd * 4 + H * hd * 4 + 2 * G * hd * 2), 0, VALU_F32)
+    # per-head products around the attention (key up-projection on the query side, value up-projection) against a dense linear of the same work
+    for T_ in (prompt, 8):
+        qn, wuk = bf(T_, H * hd), bf(H, R, hd)
+        out = f32(T_, H * dpad)
+        t = timed_k(lambda: hops.dense_grouped(qn, wuk, x_step=hd, y_step=dpad, out_dtype=torch.float32, out=out))
+        add("pokepel", "dense_grouped heads (absorb)", f"M={T_} G={H} N={R} K={hd}", t, H * R * hd * 2 + T_ * H * (hd * 2 + R * 4), 2.0 * T_ * H * R * hd, MFMA_BF16)
+        ol, wuv = bf(T_, H * R), bf(H, hd, R)
+        t = timed_k(lambda: hops.dense_grouped(ol, wuv, x_step=R, y_step=hd, out_dtype=torch.float32))
+        add("pokepel", "dense_grouped heads (values)", f"M={T_} G={H} N={hd} K={R}", t, H * R * hd * 2 + T_ * H * (R * 2 + hd * 4), 2.0 * T_ * H * R * hd, MFMA_BF16)
+        x, wd = bf(T_, H * hd), bf(R, H * hd)
+        t = timed_k(lambda: hops.dense_linear(x, wd, out_dtype=torch.float32))
+        add("nufalorn", "dense_linear", f"M={T_} N={R} K={H * hd}", t, H * R * hd * 2 + T_ * (H * hd * 2 + R * 4), 2.0 * T_ * H * R * hd, MFMA_BF16)
+    # experts: routing + sorting, both grouped linears, weighted sum, against the dense gated MLP of the same active width
+    for T_ in (prompt, 8, 1):
+        h = bf(T_, W)
+        z = f32(T_, E) * 2
+        gr = moe["router"]["groups"]
+        t = timed_k(lambda: hops.moe_align(hops.moe_route(z, gr["count"], gr["keep"], top)[0], E))
+        add("pokepel", "moe route + sort", f"T={T_} E={E} top={top}", t, T_ * (E * 4 + top * 16), 0, VALU_F32)
+        ids, wts = hops.moe_route(z, gr["count"], gr["keep"], top)
+        offs, src, place, tiles = hops.moe_align(ids, E)
+        n = T_ * top
+        used = len(set(ids.flatten().tolist()))
+        wgu = torch.stack([hops.group_gate_up(bf(fe, W), bf(fe, W)) for _ in range(E)]).contiguous()
+        t = timed_k(lambda: hops.dense_grouped(h, wgu, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=hops.ACT_SILU))
+        add("pokepel", "dense_grouped experts gated", f"M={T_}x{top} E={E} ({used} used) N={2 * fe} K={W}", t, used * 2 * fe * W * 2 + n * (W + fe) * 2, 2.0 * n * 2 * fe * W, MFMA_BF16)
+        a, wdn = bf(n, fe), bf(E, W, fe)
+        t = timed_k(lambda: hops.dense_grouped(a, wdn, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32))
+        add("pokepel", "dense_grouped experts down", f"M={T_}x{top} E={E} ({used} used) N={W} K={fe}", t, used * fe * W * 2 + n * (fe * 2 + W * 4), 2.0 * n * fe * W, MFMA_BF16)
+        y, extra = f32(n, W), f32(T_, W)
+        t = timed_k(lambda: hops.moe_combine(y, place, wts, extra))
+        add("pokepel", "moe weighted sum + shared", f"T={T_} top={top} W={W}", t, (n + 2 * T_) * W * 4, 0, VALU_F32)
+        ffa = fe * top
+        wd_gu = hops.group_gate_up(bf(ffa, W), bf(ffa, W))
+        t = timed_k(lambda: hops.dense_linear(h, wd_gu, gated=True, act=hops.ACT_RELU))
+        add("nufalorn", "dense_linear gated", f"M={T_} N={2 * ffa} K={W}", t, 2 * ffa * W * 2 + T_ * (W + ffa) * 2, 2.0 * T_ * 2 * ffa * W, MFMA_BF16)
+        wdd, aa = bf(W, ffa), bf(T_, ffa)
+        t = timed_k(lambda: hops.dense_linear(aa, wdd, out_dtype=torch.float32))
+        add("nufalorn", "dense_linear down", f"M={T_} N={W} K={ffa}", t, ffa * W * 2 + T_ * (ffa * 2 + W * 4), 2.0 * T_ * ffa * W, MFMA_BF16)
+    # PolyNorm, gated residual + norm
+    for T_ in (prompt, 8):
+        z = f32(T_, ff)
+        t = timed_k(lambda: hops.polynorm(z, (0.6, 0.3, 0.1, 0.0), 1e-6, torch.bfloat16))
+        add("pokepel", "polynorm", f"M={T_} ff={ff}", t, T_ * ff * 6, 0, VALU_F32)
+        x, a, b, gt = f32(T_, W), f32(T_, W), f32(T_, W), f32(T_, 2 * W)
+        w1, w2 = bf(W), bf(W)
+        t = timed_k(lambda: hops.residual_norm(x, a, b, 1.0, w1, None, 1e-6, gate=gt))
+        add("pokepel", "gated residual + norm (fp32 stream)", f"M={T_} W={W}", t, M_bytes(T_, W, 6, 1), 0, VALU_F32)
+        t = timed_k(lambda: hops.residual_norm(x, a, b, 0.3, w1, w2, 1e-5, weight_offset=1.0))
+        add("nufalorn", "residual + 2 norms (fp32 stream)", f"M={T_} W={W}", t, M_bytes(T_, W, 4, 2), 0, VALU_F32)
+    # recurrence: fixed decay (after the separate turn of q and k) against the gated-linear-attention scan
+    d = hd // 2
+    for T_, name in ((prompt, "prefill"), (8, "decode b=8")):
+        nseq = 1 if T_ > 8 else 8
+        proj = f32(T_, 2 * H * d + 2 * H * hd)
+        z = f32(T_, H * d)
+        rs = torch.arange(0, T_ + 1, T_ // nseq, dtype=torch.int32, device=dev)
+        slot, fp = torch.arange(nseq, dtype=torch.int32, device=dev), torch.ones(nseq, dtype=torch.int32, device=dev)
+        state = torch.zeros(nseq, H, d, hd, device=dev)
+        decay = torch.full((H,), 0.97, device=dev)
+        nb, fl = T_ * (2 * H * d + 2 * H * hd) * 4 + 2 * nseq * H * d * hd * 4, 4.0 * T_ * H * d * hd
+        t = timed_k(lambda: hops.scan(hops.SCAN_FIXED, proj, 0, H * d, 2 * H * d, None, decay, None, 1.0, 1.0, H, d, hd, rs, slot, fp, state, torch.bfloat16))
+        add("pokepel", f"scan retention {name}", f"T={T_} H={H} dim={d} vdim={hd}", t, nb, fl, VALU_F32)
+        t = timed_k(lambda: hops.scan(hops.SCAN_GLA, proj, 0, H * d, 2 * H * d, z, None, None, 16.0, d ** -0.5, H, d, hd, rs, slot, fp, state, torch.bfloat16))
+        add("nufalorn", f"scan GLA {name}", f"T={T_} H={H} dim={d} vdim={hd}", t, nb + T_ * H * d * 4, fl, VALU_F32)
+        pos = torch.arange(T_, dtype=torch.int32, device=dev)
+        fr = torch.ones(d // 2, device=dev) * 1e-3
+        t = timed_k(lambda: hops.rotary(proj, [(0, H, d, 1.0), (H * d, H, d, d ** -0.5)], d, 1, fr, 1.0, pos))
+        add("pokepel", f"rotary q, k {name}", f"T={T_} H={H} dim={d}", t, T_ * 2 * H * d * 8, 0, VALU_F32)
+    return rows
+
+
+def M_bytes(T_, W, f32_streams, bf16_streams):
+    return T_ * W * (4 * f32_streams + 2 * bf16_streams)
+
+
+def run_pokepel(args, dev, sizes):
+    prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
+    out = {}
+    for name in sizes:
+        s = SIZES[name]
+        log(f"[hybrid bench] {name}: {s}")
+        rec = {"config": s, "prompt": prompt, "batch": batch}
+        for design in ("pokepel", "nufalorn"):
+            rec[design], model, eng = bench_hybrid_engine(s, dev, prompt, batch, steps, design)
+            del model, eng
+            torch.cuda.empty_cache()
+            log(f"[hybrid bench] {name} {design}: {rec[design]}")
+        rec["kernels"] = kernel_table_pokepel(s, dev, prompt)
+        for r in rec["kernels"]:
+            log(f"    {r['family']:8s} {r['kernel']:44s} {r['shape']:48s} {r['us']:10.1f} us  roofline {r['roofline_us']:9.2f} us  x{r['x_roofline']}")
+        out[name] = rec
+    print(json.dumps({"hybrid_bench": out, "design": "pokepel", "dtype": "bf16", "data": "synthetic (random weights and tokens)"}))
+    return 0
+
+
 def run(args):
     from . import _C
     _C.lib(); _C.hybrid_lib()
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     sizes = [x for x in (args.hybrid_sizes.split(",") if args.hybrid_sizes else SIZES)]
+    if getattr(args, "hybrid_design", "nufalorn") == "pokepel":
+        return run_pokepel(args, dev, sizes)
     prompt, batch, steps = args.hybrid_prompt, args.hybrid_batch, args.steps
     out = {}
     for name in sizes:

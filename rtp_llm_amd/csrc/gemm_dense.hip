@@ -27,18 +27,25 @@ struct DenseParams {
     int vec;         // 16-byte loads allowed (alignment and K % 8 == 0 checked on the host)
     // groups (tile kernels, blockIdx.z): group g multiplies its rows by the weight w + g * ws (bias + g * N) and writes columns ys * g + ...
     // of y; it reads x from column xs * g on.  Its rows are all M rows, or rows offs[g] .. offs[g + 1] - 1 of a list sorted by group, whose
-    // entry r reads x row gather[r] (identity without gather) and writes y row r.
+    // entry r reads x row gather[r] (identity without gather) and writes y row r.  tiles (with offs): {count, (group, first row) x count}, the
+    // 64-row tiles that hold rows; blockIdx.y indexes this list instead of (blockIdx.z, row tile), so no block is spent on a tile without rows.
     int G;
     long long xs, ws, ys;
-    const int32_t* offs; const int32_t* gather;
+    const int32_t* offs; const int32_t* gather; const int32_t* tiles;
 };
 
-// rows [rbeg, rend) of the block's group and its operand bases
-struct DnGroup { int rbeg, rend; long long xo, wo, yo; int bo; };
-__device__ __forceinline__ DnGroup dn_group(const DenseParams& p) {
-    const int g = blockIdx.z;
+// first row and end of the rows of the block's tile in its group, and the group's operand bases
+struct DnGroup { int m0, rend; long long xo, wo, yo; int bo; };
+__device__ __forceinline__ DnGroup dn_group(const DenseParams& p, int tile_rows) {
+    int g = blockIdx.z;
     DnGroup r;
-    r.rbeg = p.offs ? p.offs[g] : 0; r.rend = p.offs ? p.offs[g + 1] : p.M;
+    if (p.tiles) {
+        const int i = blockIdx.y;
+        if (i >= p.tiles[0]) { r.m0 = r.rend = 0; return r; }
+        g = p.tiles[1 + 2 * i]; r.m0 = p.tiles[2 + 2 * i]; r.rend = p.offs[g + 1];
+    } else {
+        r.m0 = (p.offs ? p.offs[g] : 0) + blockIdx.y * tile_rows; r.rend = p.offs ? p.offs[g + 1] : p.M;
+    }
     r.xo = p.xs * g; r.wo = p.ws * g; r.yo = p.ys * g; r.bo = g * p.N;
     return r;
 }
@@ -80,8 +87,8 @@ __global__ __launch_bounds__(256) void dense_tile_bf16_kernel(DenseParams p) {
     __shared__ __attribute__((aligned(16))) bf16 Bs[TB_N * TB_LD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave & 1, wn = wave >> 1;                       // wave tile: rows wm*32.., cols wn*64..
-    const DnGroup gr = dn_group(p);
-    const int m0 = gr.rbeg + blockIdx.y * TB_M, n0 = blockIdx.x * TB_N;
+    const DnGroup gr = dn_group(p, TB_M);
+    const int m0 = gr.m0, n0 = blockIdx.x * TB_N;
     if (m0 >= gr.rend) return;
     const bf16* X = (const bf16*)p.x + gr.xo;
     const bf16* W = (const bf16*)p.w + gr.wo;
@@ -175,8 +182,8 @@ __global__ __launch_bounds__(256) void dense_tile_f32_kernel(DenseParams p) {
     __shared__ __attribute__((aligned(16))) float As[TF_K * TF_LD];   // [k][m]
     __shared__ __attribute__((aligned(16))) float Bs[TF_K * TF_LD];   // [k][n]
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
-    const DnGroup gr = dn_group(p);
-    const int m0 = gr.rbeg + blockIdx.y * TF_M, n0 = blockIdx.x * TF_N;
+    const DnGroup gr = dn_group(p, TF_M);
+    const int m0 = gr.m0, n0 = blockIdx.x * TF_N;
     if (m0 >= gr.rend) return;
     const float* X = (const float*)p.x + gr.xo;
     const float* W = (const float*)p.w + gr.wo;
@@ -328,6 +335,55 @@ __global__ __launch_bounds__(256) void dense_rows_kernel(DenseParams p, int mbas
     }
 }
 
+// The same for a few rows that each belong to a group of their own (the experts of a decode step): blockIdx.y is the sorted row, its group is
+// found in offs, a wave streams the weight row(s) of NC outputs of that group's weight once.
+template <typename T, int NC, bool GATED>
+__global__ __launch_bounds__(256) void dense_rows_grouped_kernel(DenseParams p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int o0 = (blockIdx.x * 4 + wave) * NC, r = blockIdx.y;
+    const int nout = GATED ? p.N / 2 : p.N;
+    if (o0 >= nout || r >= p.offs[p.G]) return;
+    int g = 0;
+    while (g + 1 < p.G && p.offs[g + 1] <= r) ++g;
+    const T* X = (const T*)p.x + (size_t)(p.gather ? p.gather[r] : r) * p.ldx + p.xs * g;
+    const T* W0[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int o = min(o0 + c, nout - 1);
+        W0[c] = (const T*)p.w + p.ws * g + (size_t)(GATED ? (o >> 5) * 64 + (o & 31) : o) * p.K;
+    }
+    float a0[NC], a1[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) a0[c] = a1[c] = 0.f;
+    for (int k = lane * 8; k < p.K; k += 64 * 8) {
+        float w0[NC][8], w1[GATED ? NC : 1][8], xv[8];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            DnVec<T>::load(W0[c] + k, p.K - k, p.vec, w0[c]);
+            if (GATED) DnVec<T>::load(W0[c] + (size_t)32 * p.K + k, p.K - k, p.vec, w1[c]);
+        }
+        DnVec<T>::load(X + k, p.K - k, p.vec, xv);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a0[c] = __builtin_fmaf(xv[i], w0[c][i], a0[c]);
+            if (GATED) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) a1[c] = __builtin_fmaf(xv[i], w1[c][i], a1[c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        float gsum = dn_wave_sum(a0[c]);
+        const float u = GATED ? dn_wave_sum(a1[c]) : 0.f;
+        const int o = o0 + c;
+        if (lane != 0 || o >= nout) continue;
+        gsum = dn_act(gsum, p.act);
+        dn_store<T>(p, r, (int)(p.ys * g) + o, GATED ? gsum * u : gsum);
+    }
+}
+
 template <typename T, bool GATED>
 void launch_rows(const DenseParams& p, hipStream_t st) {
     const int nout = GATED ? p.N / 2 : p.N;
@@ -419,7 +475,7 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
     p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr;
+    p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr; p.tiles = nullptr;
     (void)es;
     hipStream_t st = (hipStream_t)stream;
     if (bf && M > 1 && M <= 16 && p.vec) {
@@ -452,30 +508,44 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
 // bias + g * N, reads x from column xs * g on and writes y from column ys * g on.  offs null: every group takes all M rows (per-head
 // projections: xs, ys = the head's column step).  offs [G + 1] (device): M rows are sorted by group, group g owns rows offs[g] .. offs[g + 1] - 1;
 // sorted row r reads x row gather[r] (device, or null for r itself) and writes y row r (experts of a mixture: xs = ys = 0).  A row's result
-// depends on its own input and its group's weight only.
+// depends on its own input and its group's weight only.  tiles (device, with offs; null: every group is given ceil(M / 64) row tiles, most of
+// them empty): {n, (group, first row) x n}, the 64-row tiles that hold rows, at most max_tiles of them (mi355_hy_moe_align writes the list).
 extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y,
                                    int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs,
-                                   int64_t ys, const int32_t* offs, const int32_t* gather, mi355_stream_t stream) {
+                                   int64_t ys, const int32_t* offs, const int32_t* gather, const int32_t* tiles, int32_t max_tiles,
+                                   mi355_stream_t stream) {
     MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && G > 0 && xs >= 0 && ys >= 0, "dense_grouped: M=%d N=%d K=%d G=%d", M, N, K, G);
     MI355_CHECK_ARG(ldx >= xs * (G - 1) + K, "dense_grouped: ldx=%d for %d groups of K=%d at step %lld", ldx, G, K, (long long)xs);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_grouped: act_dtype=%d (bf16 or fp32)", act_dtype);
     MI355_CHECK_ARG(!gated || N % 64 == 0, "dense_grouped: gated needs N %% 64 == 0 (N=%d)", N);
     MI355_CHECK_ARG(act >= 0 && act <= 2, "dense_grouped: act=%d", act);
     MI355_CHECK_ARG(ldy >= ys * (G - 1) + (gated ? N / 2 : N), "dense_grouped: ldy=%d", ldy);
-    MI355_CHECK_ARG(G <= 65535 && (!gather || offs), "dense_grouped: G=%d, gather needs offs", G);
+    MI355_CHECK_ARG(G <= 65535 && (!gather || offs) && (!tiles || (offs && max_tiles > 0)), "dense_grouped: G=%d, gather and tiles need offs", G);
     const bool bf = act_dtype == MI355_ACT_BF16;
     DenseParams p;
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
     p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = 0.f;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && (xs % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    p.G = G; p.xs = xs; p.ws = (long long)N * K; p.ys = ys; p.offs = offs; p.gather = gather;
+    p.G = G; p.xs = xs; p.ws = (long long)N * K; p.ys = ys; p.offs = offs; p.gather = gather; p.tiles = tiles;
+    static_assert(TB_M == 64 && TF_M == 64, "the tile list is made of 64-row tiles");
     hipStream_t st = (hipStream_t)stream;
+    const int gy = tiles ? max_tiles : (M + 63) / 64, gz = tiles ? 1 : G;
+    if (offs && M <= 16 && !bias) {            // a decode step's few rows: each streams its own group's weight
+        const int nout = gated ? N / 2 : N, nc = gated ? 1 : 2;
+        const dim3 grid((nout + 4 * nc - 1) / (4 * nc), M);
+        if (bf) { if (gated) hipLaunchKernelGGL((dense_rows_grouped_kernel<bf16, 1, true>), grid, dim3(256), 0, st, p);
+                  else       hipLaunchKernelGGL((dense_rows_grouped_kernel<bf16, 2, false>), grid, dim3(256), 0, st, p); }
+        else    { if (gated) hipLaunchKernelGGL((dense_rows_grouped_kernel<float, 1, true>), grid, dim3(256), 0, st, p);
+                  else       hipLaunchKernelGGL((dense_rows_grouped_kernel<float, 2, false>), grid, dim3(256), 0, st, p); }
+        MI355_CHECK_LAUNCH("dense_rows_grouped_kernel");
+        return MI355_OK;
+    }
     if (bf) {
-        const dim3 grid((N + TB_N - 1) / TB_N, (M + TB_M - 1) / TB_M, G);
+        const dim3 grid((N + TB_N - 1) / TB_N, gy, gz);
         hipLaunchKernelGGL(dense_tile_bf16_kernel, grid, dim3(256), 0, st, p);
         MI355_CHECK_LAUNCH("dense_tile_bf16_kernel");
     } else {
-        const dim3 grid((N + TF_N - 1) / TF_N, (M + TF_M - 1) / TF_M, G);
+        const dim3 grid((N + TF_N - 1) / TF_N, gy, gz);
         hipLaunchKernelGGL(dense_tile_f32_kernel, grid, dim3(256), 0, st, p);
         MI355_CHECK_LAUNCH("dense_tile_f32_kernel");
     }

@@ -877,8 +877,10 @@ __global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld
 }
 
 // Counting sort of the n = tokens * top (token, choice) pairs by expert, one block: offs [E + 1], src_row[sorted place] = token,
-// place_of[pair] = sorted place.  The order inside an expert is arbitrary (rows are independent of each other).
-__global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, int n, int top, int E, int32_t* offs, int32_t* src_row, int32_t* place_of) {
+// place_of[pair] = sorted place, tiles = {count, (expert, first row) x count}: the 64-row tiles of the sorted list that hold rows.  The order
+// inside an expert is arbitrary (rows are independent of each other).
+__global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, int n, int top, int E, int32_t* offs, int32_t* src_row, int32_t* place_of,
+                                                            int32_t* tiles) {
     extern __shared__ int hy_cnt[];             // counts [E], cursors [E]
     int* cnt = hy_cnt;
     int* cur = hy_cnt + E;
@@ -887,9 +889,13 @@ __global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, 
     for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
     __syncthreads();
     if (threadIdx.x == 0) {
-        int a = 0;
-        for (int e = 0; e < E; ++e) { cur[e] = a; offs[e] = a; a += cnt[e]; }
-        offs[E] = a;
+        int a = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            cur[e] = a; offs[e] = a;
+            for (int m = 0; m < cnt[e]; m += 64) { tiles[1 + 2 * nt] = e; tiles[2 + 2 * nt] = a + m; ++nt; }
+            a += cnt[e];
+        }
+        offs[E] = a; tiles[0] = nt;
     }
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -1113,9 +1119,11 @@ extern "C" int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, in
     return MI355_OK;
 }
 
-extern "C" int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, int32_t E, int32_t* offs, int32_t* src_row, int32_t* place_of, mi355_stream_t stream) {
-    MI355_CHECK_ARG(ids && offs && src_row && place_of && n > 0 && top > 0 && E > 0 && (size_t)E * 8 <= 48 * 1024, "hy_moe_align: n=%d experts=%d", n, E);
-    hipLaunchKernelGGL(hy_moe_align_kernel, dim3(1), dim3(1024), (size_t)E * 8, (hipStream_t)stream, ids, n, top, E, offs, src_row, place_of);
+// tiles: int32 [1 + 2 * (n / 64 + E)] (at most n / 64 + E tiles hold rows)
+extern "C" int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, int32_t E, int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles,
+                                  mi355_stream_t stream) {
+    MI355_CHECK_ARG(ids && offs && src_row && place_of && tiles && n > 0 && top > 0 && E > 0 && (size_t)E * 8 <= 48 * 1024, "hy_moe_align: n=%d experts=%d", n, E);
+    hipLaunchKernelGGL(hy_moe_align_kernel, dim3(1), dim3(1024), (size_t)E * 8, (hipStream_t)stream, ids, n, top, E, offs, src_row, place_of, tiles);
     MI355_CHECK_LAUNCH("hy_moe_align_kernel");
     return MI355_OK;
 }

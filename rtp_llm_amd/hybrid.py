@@ -181,6 +181,11 @@ class HybridModel:
                 if mlp is None:                        # the kernel reads two gates per row: keep the row stride at 2 W
                     gate_w = torch.cat([gate_w, torch.zeros_like(gate_w)], 0).contiguous()
                     gate_b = torch.cat([gate_b, torch.zeros_like(gate_b)], 0).contiguous()
+                if isinstance(mlp, RoutedExperts):     # the router's logits come out of the same linear: columns [2W, 2W + experts), padded to 4
+                    E = L.router.experts
+                    rw = torch.cat([mlp.w_router, torch.zeros((-E) % 4, cfg.width, dtype=dtype, device=self.device)], 0)
+                    gate_w = torch.cat([gate_w, rw], 0).contiguous()
+                    gate_b = torch.cat([gate_b, torch.zeros(rw.shape[0], dtype=dtype, device=self.device)], 0).contiguous()
             n2 = get(p + "norm2") if mlp is not None and not cfg.shared_norm else None
             self.layers.append((L, mixer, mlp, get(p + "norm1"), n2, gate_w, gate_b))
         self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
@@ -228,7 +233,12 @@ class HybridModel:
                 h2 = h1
             g = hops.dense_linear(h1, gate_w, gate_b, out_dtype=torch.float32) if gate_w is not None else None
             a = mixer.forward(h1, batch, *cache) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache)
-            b = mlp.forward(h2) if mlp is not None else None
+            if mlp is None:
+                b = None
+            elif g is not None and isinstance(mlp, RoutedExperts):
+                b = mlp.forward(h2, g[:, 2 * cfg.width: 2 * cfg.width + L.router.experts])
+            else:
+                b = mlp.forward(h2)
         if collect is not None:
             hops.residual_norm(x, a, b, cfg.residual_mult, self.final_norm, None, cfg.eps, weight_offset=cfg.norm_offset, gate=g)
             collect.append(x.clone())

@@ -228,12 +228,13 @@ def head_norm(o: torch.Tensor, heads: int, vdim: int, w: Optional[torch.Tensor],
 
 
 def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: int = 0, offs: Optional[torch.Tensor] = None,
-                  gather: Optional[torch.Tensor] = None, rows: Optional[int] = None, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
+                  gather: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None, rows: Optional[int] = None, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
                   act: int = ACT_NONE, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One launch of G = w.shape[0] linears with the weights w [G, N, K].
     Without offs every group takes all rows of x, reads its K inputs from column g * x_step and writes its outputs from column g * y_step
     (per-head projections).  With offs (int32 [G + 1] on the device) the `rows` rows of the output are sorted by group, group g owns rows
-    offs[g] .. offs[g + 1] - 1, and sorted row r reads x[gather[r]] (x[r] without gather): the experts of a mixture."""
+    offs[g] .. offs[g + 1] - 1, and sorted row r reads x[gather[r]] (x[r] without gather): the experts of a mixture.  tiles: the list of
+    64-row tiles that hold rows, as moe_align writes it (without it every group is launched over all row tiles)."""
     _dev(x, w.dtype, "dense_grouped.x"); _dev(w, w.dtype, "dense_grouped.w")
     if w.dim() != 3 or not w.is_contiguous():
         raise _C.Mi355Error(f"dense_grouped: weights {tuple(w.shape)} must be contiguous [G, N, K]")
@@ -253,7 +254,7 @@ def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: 
             raise _C.Mi355Error(f"dense_grouped: out {tuple(out.shape)} for [{M}, {width}]")
     if x.shape[1] < x_step * (G - 1) + K:
         raise _C.Mi355Error(f"dense_grouped: x {tuple(x.shape)} for {G} groups of K={K} at step {x_step}")
-    for t, nm in ((offs, "offs"), (gather, "gather")):
+    for t, nm in ((offs, "offs"), (gather, "gather"), (tiles, "tiles")):
         if t is not None:
             _dev(t, torch.int32, "dense_grouped." + nm)
     if offs is not None and offs.numel() != G + 1:
@@ -263,7 +264,8 @@ def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: 
     if M:
         _C.check_hybrid(_C.hybrid_lib().mi355_dense_grouped(x.data_ptr(), ldx, M, w.data_ptr(), N, K, None, out.data_ptr(), _rows(out, "dense_grouped.out"),
                                                             1 if od == torch.float32 else 0, 1 if gated else 0, act, act_code(w.dtype), G, x_step, y_step,
-                                                            _p(offs), _p(gather), _stream()), "dense_grouped")
+                                                            _p(offs), _p(gather), _p(tiles), 0 if tiles is None else (tiles.numel() - 1) // 2, _stream()),
+                        "dense_grouped")
     return out
 
 
@@ -342,17 +344,19 @@ def moe_route(z: torch.Tensor, groups: int, keep: int, top: int):
 
 
 def moe_align(ids: torch.Tensor, experts: int):
-    """ids int32 [T, top] -> (offs int32 [E + 1], src_row int32 [T * top], place_of int32 [T * top]): the (token, choice) pairs sorted by
-    expert; sorted place p belongs to token src_row[p], pair i sits at place_of[i]."""
+    """ids int32 [T, top] -> (offs int32 [E + 1], src_row int32 [T * top], place_of int32 [T * top], tiles): the (token, choice) pairs sorted
+    by expert; sorted place p belongs to token src_row[p], pair i sits at place_of[i]; tiles = {count, (expert, first row) x count} lists the
+    64-row tiles of the sorted rows for dense_grouped."""
     _dev(ids, torch.int32, "moe_align.ids")
     T, top = ids.shape
     offs = torch.empty(experts + 1, dtype=torch.int32, device=ids.device)
     src = torch.empty(T * top, dtype=torch.int32, device=ids.device)
     place = torch.empty(T * top, dtype=torch.int32, device=ids.device)
+    tiles = torch.empty(1 + 2 * (T * top // 64 + experts), dtype=torch.int32, device=ids.device)
     if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_align(ids.data_ptr(), T * top, top, experts, offs.data_ptr(), src.data_ptr(), place.data_ptr(), _stream()),
-                        "hy_moe_align")
-    return offs, src, place
+        _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_align(ids.data_ptr(), T * top, top, experts, offs.data_ptr(), src.data_ptr(), place.data_ptr(),
+                                                           tiles.data_ptr(), _stream()), "hy_moe_align")
+    return offs, src, place, tiles
 
 
 def moe_combine(y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -365,13 +365,16 @@ class RoutedExperts:
         self.w_gate_up, self.w_down = torch.stack(gu).contiguous(), torch.stack(dn).contiguous()
         self.shared, self.act = shared, hops.ACTIVATIONS[act]
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """logits: the router's fp32 logits [T, experts] when the caller has computed them (in a linear shared with other projections of h)."""
         r = self.router
-        ids, wts = hops.moe_route(hops.dense_linear(h, self.w_router, out_dtype=torch.float32), r.groups, r.keep, r.top)
-        offs, src, place = hops.moe_align(ids, r.experts)
+        if logits is None:
+            logits = hops.dense_linear(h, self.w_router, out_dtype=torch.float32)
+        ids, wts = hops.moe_route(logits, r.groups, r.keep, r.top)
+        offs, src, place, tiles = hops.moe_align(ids, r.experts)
         n = ids.numel()
-        a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, rows=n, gated=True, act=self.act)
-        y = hops.dense_grouped(a, self.w_down, offs=offs, rows=n, out_dtype=torch.float32)
+        a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=self.act)
+        y = hops.dense_grouped(a, self.w_down, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32)
         return hops.moe_combine(y, place, wts, self.shared.forward(h) if self.shared is not None else None)
 
 

@@ -56,25 +56,28 @@ def test_grouped_linear_heads_and_sorted_rows():
                 close(y[:, j * (N + 3):j * (N + 3) + N], (x[:, j * K:(j + 1) * K].double() @ w[j].double().T).cpu(), tol)
         # rows sorted by group with a gather on the input, empty groups, groups larger than a tile; gated epilogue
         E, K, ff, T = 6, 40, 32, 90
-        counts = [0, 75, 1, 0, 130, 3]
-        n = sum(counts)
-        offs = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
-        src = torch.randint(0, T, (n,), generator=torch.Generator().manual_seed(2)).to(torch.int32).to(DEV)
-        x = torch.randn(T, K, device=DEV, generator=g).to(dt)
-        gt, up = [(torch.randn(E, ff, K, device=DEV, generator=g) * 0.2).to(dt) for _ in range(2)]
-        wgu = torch.stack([hops.group_gate_up(gt[e], up[e]) for e in range(E)]).contiguous()
-        a = hops.dense_grouped(x, wgu, offs=offs, gather=src, rows=n, gated=True, act=hops.ACT_SILU, out_dtype=torch.float32)
-        wd = (torch.randn(E, 24, ff, device=DEV, generator=g) * 0.2).to(dt)
-        xs = torch.randn(n, ff, device=DEV, generator=g).to(dt)
-        y = hops.dense_grouped(xs, wd, offs=offs, rows=n, out_dtype=torch.float32)
-        at = 0
-        for e, c in enumerate(counts):
-            if not c:
-                continue
-            xe = x[src[at:at + c].long()].double()
-            close(a[at:at + c], (torch.nn.functional.silu(xe @ gt[e].double().T) * (xe @ up[e].double().T)).cpu(), tol)
-            close(y[at:at + c], (xs[at:at + c].double() @ wd[e].double().T).cpu(), tol)
-            at += c
+        for counts in ([0, 75, 1, 0, 130, 3], [0, 2, 1, 0, 5, 3], [0, 0, 0, 1, 0, 0]):      # prompt-sized, and the few rows of a decode step
+            n = sum(counts)
+            offs = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
+            src = torch.randint(0, T, (n,), generator=torch.Generator().manual_seed(2)).to(torch.int32).to(DEV)
+            x = torch.randn(T, K, device=DEV, generator=g).to(dt)
+            gt, up = [(torch.randn(E, ff, K, device=DEV, generator=g) * 0.2).to(dt) for _ in range(2)]
+            wgu = torch.stack([hops.group_gate_up(gt[e], up[e]) for e in range(E)]).contiguous()
+            a = hops.dense_grouped(x, wgu, offs=offs, gather=src, rows=n, gated=True, act=hops.ACT_SILU, out_dtype=torch.float32)
+            wd = (torch.randn(E, 24, ff, device=DEV, generator=g) * 0.2).to(dt)
+            xs = torch.randn(n, ff, device=DEV, generator=g).to(dt)
+            y = hops.dense_grouped(xs, wd, offs=offs, rows=n, out_dtype=torch.float32)
+            tl = [(e, m) for e in range(E) for m in range(int(offs[e]), int(offs[e + 1]), 64)]
+            tiles = torch.tensor([len(tl)] + [v for pr in tl for v in pr] + [0, 0], dtype=torch.int32, device=DEV)      # the same through a tile list
+            assert torch.equal(y, hops.dense_grouped(xs, wd, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32))
+            at = 0
+            for e, c in enumerate(counts):
+                if not c:
+                    continue
+                xe = x[src[at:at + c].long()].double()
+                close(a[at:at + c], (torch.nn.functional.silu(xe @ gt[e].double().T) * (xe @ up[e].double().T)).cpu(), tol)
+                close(y[at:at + c], (xs[at:at + c].double() @ wd[e].double().T).cpu(), tol)
+                at += c
 
 
 def test_gated_branches_join_the_stream():
@@ -113,8 +116,10 @@ def test_router_choices_and_weights(E, groups, keep, top):
     want_ids, want_w = O.route(z.double(), {"r.router": torch.eye(E, dtype=torch.float64)}, "r.", router)       # identity router: logits = z
     assert torch.equal(ids.cpu().long(), want_ids)
     close(wts, want_w, 1e-6)
-    offs, src, place = hops.moe_align(ids, E)
-    offs, src, place = offs.cpu(), src.cpu(), place.cpu()
+    offs, src, place, tiles = hops.moe_align(ids, E)
+    offs, src, place, tiles = offs.cpu(), src.cpu(), place.cpu(), tiles.cpu().tolist()
+    want_tiles = [(e, m) for e in range(E) for m in range(int(offs[e]), int(offs[e + 1]), 64)]
+    assert tiles[0] == len(want_tiles) and list(zip(tiles[1:1 + 2 * tiles[0]:2], tiles[2:2 + 2 * tiles[0]:2])) == want_tiles
     flat = ids.cpu().flatten()
     assert offs[0] == 0 and offs[-1] == flat.numel() and sorted(place.tolist()) == list(range(flat.numel()))
     for i, e in enumerate(flat.tolist()):
