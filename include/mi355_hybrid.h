@@ -27,7 +27,7 @@ int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t voff, const
                        void* kcache, void* vcache, int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                        const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
-                       const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);
+                       const void* vcache, void* out, int32_t splits, float* parts, int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                         const int32_t* pos, const int32_t* seq, const int32_t* block_table, const int32_t* tile_row0, const int32_t* tile_n,
                         int32_t tiles, const void* kcache, const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream);

@@ -169,7 +169,7 @@ HYBRID_SIGNATURES = {
     "mi355_hy_embed": (i32, [vp, i32, vp, i32, i32, vp, i32, vp]),
     "mi355_hy_residual_norm": (i32, [vp, vp, vp, f32, vp, i32, i32, vp, vp, f32, f32, vp, vp, i32, vp]),
     "mi355_hy_attn_prep": (i32, [vp, i32, i32, i32, ip, vp, vp, i32, f32, vp, vp, vp, i32, vp, vp, i32, vp]),
-    "mi355_hy_attn_rows": (i32, [vp, i32, f32, ip, i32, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp]),
+    "mi355_hy_attn_rows": (i32, [vp, i32, f32, ip, i32, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, vp]),
     "mi355_hy_attn_tiles": (i32, [vp, i32, f32, ip, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp]),
     "mi355_hy_scan": (i32, [i32, vp, i32, i32, i32, i32, vp, i32, vp, vp, f32, f32, i32, i32, i32, vp, vp, vp, i32, vp, vp, i32, vp]),
     "mi355_hy_head_norm": (i32, [vp, i32, i32, i32, vp, f32, vp, i32, i32, vp, i32, vp]),

@@ -19,6 +19,24 @@ template <> __device__ __forceinline__ void hy_load8<float>(const float* p, floa
     for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
 }
 
+// eight consecutive cache elements as loaded (16 bytes of bf16, 32 of fp32), widened only where they are used: more loads fit in flight
+template <typename T> struct HyRaw8;
+template <> struct HyRaw8<bf16> {
+    u32x4 r;
+    __device__ __forceinline__ void load(const bf16* p) { r = *(const u32x4*)p; }
+    __device__ __forceinline__ void zero() { r = u32x4{0u, 0u, 0u, 0u}; }
+    __device__ __forceinline__ void get(float (&o)[8]) const { act_unpack8<true>(r, o); }
+};
+template <> struct HyRaw8<float> {
+    f32x4 a, b;
+    __device__ __forceinline__ void load(const float* p) { a = *(const f32x4*)p; b = *(const f32x4*)(p + 4); }
+    __device__ __forceinline__ void zero() { a = b = f32x4{0.f, 0.f, 0.f, 0.f}; }
+    __device__ __forceinline__ void get(float (&o)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
+    }
+};
+
 __device__ __forceinline__ float hy_wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -188,15 +206,16 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
 // ------------------------------------------------------------------------------------------------ attention over the paged cache
 constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
 
-// Four waves per (row, head): wave w takes the 64-key tiles w, w + 4, ... of the row's visible range with its own running maximum,
-// denominator and value sum; the four are merged at the end.  Inside a tile a lane scores one key (its whole q . k), the tile's weights and
-// page rows then travel by lane broadcast (uniform loop index -> v_readlane), and a lane accumulates its own value channels over the keys.
+// Four or sixteen waves per (row, head): wave w takes the 64-key tiles w, w + NW, ... of the row's visible range with its own running maximum,
+// denominator and value sum; they are merged at the end.  Inside a tile a lane owns one key; the scores are computed by groups of lanes that
+// share a key row (whole rows per load instruction: the address unit sees each cache line once), the weights and page rows then travel by
+// lane broadcast, and groups of lanes accumulate the value channels of whole value rows in the same way.
 __device__ __forceinline__ float hy_lane_f(float v, int j) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), j)); }
 
 template <typename T>
 __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
-                                                           const T* kcache, const T* vcache, T* out) {
+                                                           const T* kcache, const T* vcache, T* out, float* parts) {
     constexpr int NV = HY_MAX_VDIM / 64;
     __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
     __shared__ float m_s[16], l_s[16];
@@ -204,13 +223,14 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     __shared__ float part_s[16][64][8];
     __shared__ float o_s[HY_MAX_VDIM];
     const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NW = blockDim.x >> 6, NT = blockDim.x;
+    const int S = gridDim.z, sp = blockIdx.z;             // the row's key tiles are dealt over S blocks; with S > 1 they leave partial sums
     const int p = __builtin_amdgcn_readfirstlane(pos[r]), kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r] * g.max_blocks;
     for (int d = tid; d < g.dim; d += NT) q_s[d] = q[(size_t)r * ldq + h * g.dim + d];
     __syncthreads();
     const int lo = chunk > 0 ? (p / chunk) * chunk : 0;
     // the sink is a key of (unscaled) score sink[h] that carries no value: wave 0 starts from m = sink[h], l = 1
-    float m = (sink && wave == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0) ? 1.f : 0.f;
+    float m = (sink && wave == 0 && sp == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0 && sp == 0) ? 1.f : 0.f;
     float acc[NV], facc[8];
 #pragma unroll
     for (int i = 0; i < NV; ++i) acc[i] = 0.f;
@@ -220,31 +240,52 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 256: KPI >= 2)
     const int grp = lane / LPK, cl = (lane % LPK) * 8;
     const bool gok = grp < KPI;
-    for (int t0 = lo + wave * 64; t0 <= p; t0 += 64 * NW) {
+    // the same for the keys: LK lanes per key row (a power of two >= dim / 8), KK keys per load instruction
+    const bool coop = g.dim % 8 == 0;
+    int LK = 1;
+    while (LK * 8 < g.dim) LK <<= 1;
+    const int KK = 64 / LK, kg = lane / LK, kl = lane % LK;
+    const bool kl_ok = kl * 8 < g.dim;
+    float qv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qv[i] = (coop && kl_ok) ? q_s[kl * 8 + i] : 0.f;
+    for (int t0 = lo + (sp * NW + wave) * 64; t0 <= p; t0 += 64 * NW * S) {
         const int kj = t0 + lane;
         const bool valid = kj <= p;
         float s = -INFINITY;
         int rowi = 0;                                              // row of the key inside the cache tensors: (page * G + kv head) * page size + offset
-        if (valid) {
-            rowi = (bt[kj / g.page] * g.G + kvh) * g.page + (kj % g.page);
+        if (valid) rowi = (bt[kj / g.page] * g.G + kvh) * g.page + (kj % g.page);
+        if (coop) {
+            // LK lanes share a key row (8 channels = one 16- or 32-byte piece each), so a load instruction reads KK whole rows instead of one
+            // piece of 64 rows; the partial products are summed over the LK lanes and handed to the lane that owns the key
+            const int nk = min(64, p - t0 + 1);
+            float sc = 0.f;
+            constexpr int UB = 8;                                  // load instructions in flight
+            for (int it0 = 0; it0 * KK < nk; it0 += UB) {
+                HyRaw8<T> kr[UB];
+#pragma unroll
+                for (int u = 0; u < UB; ++u) {
+                    const int key = (it0 + u) * KK + kg;
+                    const int rk = __shfl(rowi, key & 63, 64);
+                    if (kl_ok && key < nk) kr[u].load(kcache + (size_t)rk * g.dim + kl * 8);
+                    else kr[u].zero();
+                }
+#pragma unroll
+                for (int u = 0; u < UB; ++u) {
+                    float kv[8], part = 0.f;
+                    kr[u].get(kv);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) part = __builtin_fmaf(qv[i], kv[i], part);
+                    for (int o = LK >> 1; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+                    const float got = __shfl(part, (lane % KK) * LK, 64);
+                    if (lane / KK == it0 + u) sc = got;
+                }
+            }
+            if (valid) s = sc * scale;
+        } else if (valid) {
             const T* kp = kcache + (size_t)rowi * g.dim;
             float d0 = 0.f;
-            if (g.dim % 8 == 0) {
-                for (int d = 0; d < g.dim; d += 64) {              // eight 16-byte pieces of the key row in flight
-                    float kv[8][8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (d + 8 * u < g.dim) hy_load8<T>(kp + d + 8 * u, kv[u]);
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        if (d + 8 * u < g.dim) {
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) d0 = __builtin_fmaf(q_s[d + 8 * u + i], kv[u][i], d0);
-                        }
-                }
-            } else {
-                for (int d = 0; d < g.dim; ++d) d0 = __builtin_fmaf(q_s[d], (float)kp[d], d0);
-            }
+            for (int d = 0; d < g.dim; ++d) d0 = __builtin_fmaf(q_s[d], (float)kp[d], d0);
             s = d0 * scale;
         }
         const float mn = fmaxf(m, hy_wave_max(s));
@@ -257,25 +298,27 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
             // LPK lanes share one key's value row (8 channels = 16 bytes each), so one load instruction covers KPI keys
 #pragma unroll
             for (int i = 0; i < 8; ++i) facc[i] *= corr;
-            for (int j = 0; j < nv; j += 4 * KPI) {
-                float pw[4], vv[4][8];
+            constexpr int VF = sizeof(T) == 2 ? 8 : 4;             // value pieces in flight per lane
+            for (int j = 0; j < nv; j += VF * KPI) {
+                float pw[VF];
+                HyRaw8<T> vr[VF];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < VF; ++u) {
                     const int kk = j + u * KPI + grp;
                     const bool ok = gok && kk < nv;
                     const float pk = __shfl(pj, kk & 63, 64);
                     const int rk = __shfl(rowi, kk & 63, 64);
                     pw[u] = ok ? pk : 0.f;
-                    if (ok) hy_load8<T>(vcache + (size_t)rk * g.v_ld + cl, vv[u]);
-                    else {
-#pragma unroll
-                        for (int i = 0; i < 8; ++i) vv[u][i] = 0.f;
-                    }
+                    if (ok) vr[u].load(vcache + (size_t)rk * g.v_ld + cl);
+                    else vr[u].zero();
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
+                for (int u = 0; u < VF; ++u) {
+                    float vv[8];
+                    vr[u].get(vv);
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) facc[i] = __builtin_fmaf(pw[u], vv[u][i], facc[i]);
+                    for (int i = 0; i < 8; ++i) facc[i] = __builtin_fmaf(pw[u], vv[i], facc[i]);
+                }
             }
         } else {
 #pragma unroll
@@ -312,13 +355,19 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     for (int w = 1; w < NW; ++w) mm = fmaxf(mm, m_s[w]);
     float lt = 0.f;
     for (int w = 0; w < NW; ++w) lt = __builtin_fmaf(l_s[w], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), lt);
-    const float invl = lt > 0.f ? 1.f / lt : 0.f;
+    const float invl = S > 1 ? 1.f : (lt > 0.f ? 1.f / lt : 0.f);
     for (int c = tid; c < g.vdim; c += NT) {
         float a = 0.f;
         for (int w = 0; w < NW; ++w) a = __builtin_fmaf(acc_s[w][c], (m_s[w] == -INFINITY) ? 0.f : expf(m_s[w] - mm), a);
         o_s[c] = a * invl;
     }
     __syncthreads();
+    if (S > 1) {        // partial of this block: {running maximum, denominator, value sums}; hy_attn_merge_kernel finishes the row
+        float* pd = parts + (((size_t)r * g.H + h) * S + sp) * (g.vdim + 2);
+        if (tid == 0) { pd[0] = mm; pd[1] = lt; }
+        for (int c = tid; c < g.vdim; c += NT) pd[2 + c] = o_s[c];
+        return;
+    }
     T* od = out + ((size_t)r * g.H + h) * g.vdim;
     if (vfreq) {     // turn the summed values back by the query's own position
         const float fp = (float)p;
@@ -332,6 +381,45 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
         }
     } else {
         for (int c = tid; c < g.vdim; c += NT) od[c] = (T)o_s[c];
+    }
+}
+
+// The S partials of a (row, head) -> the head's output: common maximum, summed denominators, value sums rescaled, then the turn back.
+template <typename T>
+__global__ __launch_bounds__(256) void hy_attn_merge_kernel(const float* parts, int S, AttnGeom g, const float* vfreq, const int32_t* pos, T* out) {
+    __shared__ float o_s[HY_MAX_VDIM];
+    const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const float* pd = parts + ((size_t)r * g.H + h) * S * (g.vdim + 2);
+    float mm = -INFINITY;
+    for (int s_ = 0; s_ < S; ++s_) mm = fmaxf(mm, pd[(size_t)s_ * (g.vdim + 2)]);
+    float lt = 0.f;
+    for (int s_ = 0; s_ < S; ++s_) {
+        const float ms = pd[(size_t)s_ * (g.vdim + 2)];
+        lt = __builtin_fmaf(pd[(size_t)s_ * (g.vdim + 2) + 1], (ms == -INFINITY) ? 0.f : expf(ms - mm), lt);
+    }
+    const float invl = lt > 0.f ? 1.f / lt : 0.f;
+    for (int c = tid; c < g.vdim; c += 256) {
+        float a = 0.f;
+        for (int s_ = 0; s_ < S; ++s_) {
+            const float ms = pd[(size_t)s_ * (g.vdim + 2)];
+            a = __builtin_fmaf(pd[(size_t)s_ * (g.vdim + 2) + 2 + c], (ms == -INFINITY) ? 0.f : expf(ms - mm), a);
+        }
+        o_s[c] = a * invl;
+    }
+    __syncthreads();
+    T* od = out + ((size_t)r * g.H + h) * g.vdim;
+    if (vfreq) {
+        const float fp = (float)pos[r];
+        for (int mi = tid; mi < g.vdim / 2; mi += 256) {
+            int c0, c1;
+            hy_pair(g.v_layout, mi, g.vdim, c0, c1);
+            float sn, cs;
+            sincosf(fp * vfreq[mi], &sn, &cs);
+            const float a = o_s[c0], b = o_s[c1];
+            od[c0] = (T)(a * cs + b * sn); od[c1] = (T)(b * cs - a * sn);
+        }
+    } else {
+        for (int c = tid; c < g.vdim; c += 256) od[c] = (T)o_s[c];
     }
 }
 
@@ -987,17 +1075,24 @@ extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t 
 }
 
 // out [rows, H * vdim] of act_dtype.  chunk > 0: row at position i sees keys j <= i of its own block of `chunk` positions; 0: all j <= i.
+// splits > 1 (few rows with long contexts): the key tiles of a row are dealt over `splits` blocks that leave partial sums in parts
+// (fp32 [rows, H, splits, vdim + 2]) and a second launch merges them; splits == 1 needs no parts.
 // sink: null, or fp32 [H]: exp(sink[h]) is added to head h's softmax denominator (a key of that unscaled score without a value).  vfreq non-null: the head output is turned back by the row's position.
 extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, const int32_t* geom, int32_t chunk, const float* sink, const float* vfreq,
                                   const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, const void* kcache,
-                                  const void* vcache, void* out, int32_t act_dtype, mi355_stream_t stream) {
+                                  const void* vcache, void* out, int32_t splits, float* parts, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
+    MI355_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || parts), "hy_attn_rows: %d splits", splits);
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     const int threads = rows * g.H <= 2048 ? 1024 : 256;     // few (decode) rows: sixteen waves share a row's keys
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H), dim3(threads), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
-                                              pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out));
+    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_rows_kernel<T>, dim3(rows, g.H, splits), dim3(threads), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, sink, vfreq,
+                                              pos, seq, block_table, (const T*)kcache, (const T*)vcache, (T*)out, parts));
     MI355_CHECK_LAUNCH("hy_attn_rows_kernel");
+    if (splits > 1) {
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_merge_kernel<T>, dim3(rows, g.H), dim3(256), 0, (hipStream_t)stream, parts, splits, g, vfreq, pos, (T*)out));
+        MI355_CHECK_LAUNCH("hy_attn_merge_kernel");
+    }
     return MI355_OK;
 }
 

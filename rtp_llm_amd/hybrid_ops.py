@@ -166,14 +166,21 @@ def _sink(sink: Optional[torch.Tensor], heads: int):
 def attn_rows(q: torch.Tensor, scale: float, geom, chunk: int, sink: Optional[torch.Tensor], vfreq, pos, seq, block_table, kcache, vcache,
               heads: int, vdim: int):
     """Attention of every row over its sequence's pages -> [T, heads * vdim] in the cache dtype.  sink: fp32 [heads] or None; exp(sink[h])
-    joins head h's softmax denominator."""
+    joins head h's softmax denominator.  Few rows over long block tables (decode steps) are dealt over several blocks per (row, head) whose
+    partial sums a second launch merges; the count depends on the rows and the table's width only."""
     _dev(q, torch.float32, "attn_rows.q")
     T = q.shape[0]
     out = torch.empty(T, heads * vdim, dtype=kcache.dtype, device=q.device)
+    splits, parts = 1, None
+    if chunk == 0 and T * heads <= 2048:                   # sixteen waves per block: one 64-key tile per wave and block where the chip has room
+        tiles = (block_table.shape[1] * geom[7] + 63) // 64
+        splits = max(1, min(16, (tiles + 15) // 16, 1024 // (T * heads)))
+        if splits > 1:
+            parts = torch.empty(T * heads * splits * (vdim + 2), dtype=torch.float32, device=q.device)
     if T:
         _C.check_hybrid(_C.hybrid_lib().mi355_hy_attn_rows(q.data_ptr(), _rows(q, "attn_rows.q"), float(scale), geom, int(chunk), _sink(sink, heads), _p(vfreq),
                                                            pos.data_ptr(), seq.data_ptr(), block_table.data_ptr(), T, kcache.data_ptr(), vcache.data_ptr(),
-                                                           out.data_ptr(), act_code(kcache.dtype), _stream()), "hy_attn_rows")
+                                                           out.data_ptr(), splits, _p(parts), act_code(kcache.dtype), _stream()), "hy_attn_rows")
     return out
 
 
