@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void hy_attn_prep_kernel(float* qkv, int ld, i
 }
 
 // ------------------------------------------------------------------------------------------------ attention over the paged cache
-constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 256;
+constexpr int HY_MAX_DIM = 512, HY_MAX_VDIM = 512;
 
 // Four or sixteen waves per (row, head): wave w takes the 64-key tiles w, w + NW, ... of the row's visible range with its own running maximum,
 // denominator and value sum; they are merged at the end.  Inside a tile a lane owns one key; the scores are computed by groups of lanes that
@@ -220,7 +220,6 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
     __shared__ __attribute__((aligned(16))) float q_s[HY_MAX_DIM];
     __shared__ float m_s[16], l_s[16];
     __shared__ float acc_s[16][HY_MAX_VDIM];
-    __shared__ float part_s[16][64][8];
     __shared__ float o_s[HY_MAX_VDIM];
     const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, NW = blockDim.x >> 6, NT = blockDim.x;
     const int S = gridDim.z, sp = blockIdx.z;             // the row's key tiles are dealt over S blocks; with S > 1 they leave partial sums
@@ -237,7 +236,7 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
 #pragma unroll
     for (int i = 0; i < 8; ++i) facc[i] = 0.f;
     const bool fast = g.vdim % 8 == 0 && g.v_ld % 8 == 0;
-    const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 256: KPI >= 2)
+    const int LPK = fast ? g.vdim / 8 : 1, KPI = fast ? 64 / LPK : 1;      // lanes per key, keys per load instruction (vdim <= 512: KPI >= 1)
     const int grp = lane / LPK, cl = (lane % LPK) * 8;
     const bool gok = grp < KPI;
     // the same for the keys: LK lanes per key row (a power of two >= dim / 8), KK keys per load instruction
@@ -336,14 +335,17 @@ __global__ __launch_bounds__(1024) void hy_attn_rows_kernel(const float* q, int 
             }
         }
     }
-    if (fast) {       // sum the KPI partial rows of this wave into acc_s[wave]
+    if (fast) {       // sum the KPI partial rows of this wave (lanes j, j + LPK, ...) into acc_s[wave]
+        float tot[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) part_s[wave][lane][i] = facc[i];
-        __syncthreads();
-        for (int c = lane; c < g.vdim; c += 64) {
-            float a = 0.f;
-            for (int k = 0; k < KPI; ++k) a += part_s[wave][k * LPK + (c >> 3)][c & 7];
-            acc_s[wave][c] = a;
+        for (int i = 0; i < 8; ++i) tot[i] = facc[i];
+        for (int k = 1; k < KPI; ++k) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tot[i] += __shfl(facc[i], (lane + k * LPK) & 63, 64);
+        }
+        if (lane < LPK) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc_s[wave][lane * 8 + i] = tot[i];
         }
     } else {
 #pragma unroll
@@ -1007,7 +1009,7 @@ __global__ __launch_bounds__(256) void hy_moe_combine_kernel(const float* y, int
 int hy_geom_ok(const AttnGeom& g) {
     MI355_CHECK_ARG(g.H > 0 && g.G > 0 && g.H % g.G == 0, "hybrid attention: heads=%d kv_heads=%d", g.H, g.G);
     MI355_CHECK_ARG(g.dim > 0 && g.dim <= HY_MAX_DIM, "hybrid attention: head size %d (<= %d)", g.dim, HY_MAX_DIM);
-    MI355_CHECK_ARG(g.vdim > 0 && g.vdim % 2 == 0 && g.vdim <= HY_MAX_VDIM, "hybrid attention: value size %d (even, <= %d)", g.vdim, HY_MAX_VDIM);
+    MI355_CHECK_ARG(g.vdim > 0 && g.vdim <= HY_MAX_VDIM, "hybrid attention: value size %d (<= %d)", g.vdim, HY_MAX_VDIM);
     MI355_CHECK_ARG(g.rot_dims >= 0 && g.rot_dims <= g.dim && g.rot_dims % 2 == 0, "hybrid attention: rotary span %d of %d", g.rot_dims, g.dim);
     MI355_CHECK_ARG(g.page > 0 && g.max_blocks > 0 && g.num_pages > 0, "hybrid attention: page=%d max_blocks=%d pages=%d", g.page, g.max_blocks, g.num_pages);
     MI355_CHECK_ARG(g.v_ld >= g.vdim, "hybrid attention: value row stride %d under the value size %d", g.v_ld, g.vdim);
@@ -1068,6 +1070,7 @@ extern "C" int mi355_hy_attn_prep(float* qkv, int32_t ld, int32_t koff, int32_t 
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     MI355_CHECK_ARG((g.rot_dims == 0 || kfreq) && (!kcache || (vcache && block_table)), "hy_attn_prep: missing table or cache");
+    MI355_CHECK_ARG(!vfreq || g.vdim % 2 == 0, "hy_attn_prep: rotated values need an even value size (%d)", g.vdim);
     HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_attn_prep_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, qkv, ld, koff, voff, g, kfreq, vfreq,
                                               v_norm, eps, pos, seq, block_table, (T*)kcache, (T*)vcache));
     MI355_CHECK_LAUNCH("hy_attn_prep_kernel");
@@ -1083,6 +1086,7 @@ extern "C" int mi355_hy_attn_rows(const float* q, int32_t ldq, float scale, cons
                                   const void* vcache, void* out, int32_t splits, float* parts, int32_t act_dtype, mi355_stream_t stream) {
     MI355_CHECK_ARG(q && geom && pos && seq && block_table && kcache && vcache && out && rows > 0 && chunk >= 0, "hy_attn_rows: bad argument");
     MI355_CHECK_ARG(splits >= 1 && splits <= 64 && (splits == 1 || parts), "hy_attn_rows: %d splits", splits);
+    MI355_CHECK_ARG(!vfreq || geom[3] % 2 == 0, "hy_attn_rows: rotated values need an even value size (%d)", geom[3]);
     const AttnGeom g{geom[0], geom[1], geom[2], geom[3], geom[4], geom[5], geom[6], geom[7], geom[8], geom[9], geom[10] > 0 ? geom[10] : geom[3]};
     if (int e = hy_geom_ok(g)) return e;
     const int threads = rows * g.H <= 2048 ? 1024 : 256;     // few (decode) rows: sixteen waves share a row's keys

@@ -133,6 +133,8 @@ ALONE = {
     "latent_one_head_rank_not_of_8": U.latent_layer(heads=1, dim=12, rot_dim=6, vdim=10, kv_rank=22),
     "latent_row_fills_its_padding": U.latent_layer(heads=4, dim=8, rot_dim=16, vdim=72, kv_rank=48),
     "latent_wide_rank": U.latent_layer(heads=2, dim=40, rot_dim=32, vdim=16, kv_rank=200),
+    "latent_rank_over_256": U.latent_layer(heads=2, dim=16, rot_dim=16, vdim=16, kv_rank=336),
+    "latent_odd_rank": U.latent_layer(heads=3, dim=8, rot_dim=8, vdim=12, kv_rank=27),
     "latent_no_rotated_part_scaled": U.latent_layer(heads=5, dim=16, rot_dim=2, vdim=16, kv_rank=16, scale=0.5),
     "retention": U.retention_layer(),
     "retention_partial_rotary": U.retention_layer(heads=3, dim=24, vdim=16, rot_dims=8),
