@@ -454,7 +454,7 @@ constexpr int AT_LD = 40;     // LDS row stride (elements) of the 32-key tiles: 
 template <int DKM, int NCBM, int NWV>     // most 32-channel steps of a key row / 16-channel fragments of a value row the instance holds; waves per block
 __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int ldq, float scale, AttnGeom g, int chunk, const float* sink, const float* vfreq,
                                                            const int32_t* pos, const int32_t* seq, const int32_t* block_table,
-                                                           const int32_t* tile_row0, const int32_t* tile_n, const bf16* kcache, const bf16* vcache,
+                                                           const int32_t* tile_row0, const int32_t* tile_n, int ntiles, const bf16* kcache, const bf16* vcache,
                                                            bf16* out) {
     __shared__ __attribute__((aligned(16))) bf16 Ph_all[4][16 * AT_LD];
     __shared__ __attribute__((aligned(16))) bf16 Pl_all[4][16 * AT_LD];
@@ -462,9 +462,14 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
     // the waves of a block are query heads that share one key/value head: they walk the same keys and share the transposed value tile
     const int wave = threadIdx.x >> 6;
     constexpr int VEM = NCBM / NWV;                           // 32 VP pieces of 16 bytes over 64 NWV threads: at most NCBM / NWV per thread
-    const int tile = blockIdx.x, h = blockIdx.y * NWV + wave, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
+    const int h = blockIdx.y * NWV + wave, lane = threadIdx.x & 63, lr = lane & 15, lq = lane >> 4;
     bf16* Ph = Ph_all[wave];
     bf16* Pl = Pl_all[wave];
+    // a block takes tile b and then tile ntiles - 1 - b: under a causal mask an early (short) tile of a prompt and a late (long) one, so that
+    // the blocks of one prompt walk about the same number of keys
+    for (int pass = 0; pass < 2; ++pass) {
+    const int tile = pass == 0 ? (int)blockIdx.x : ntiles - 1 - (int)blockIdx.x;
+    if (pass == 1 && tile <= (int)blockIdx.x) break;
     const int r0 = tile_row0[tile], n = tile_n[tile];
     const int p0 = pos[r0], kvh = h / (g.H / g.G);
     const int32_t* bt = block_table + (size_t)seq[r0] * g.max_blocks;
@@ -617,6 +622,7 @@ __global__ __launch_bounds__(256) void hy_attn_tiles_kernel(const float* q, int 
             if (row < n) od[c] = (bf16)v;
         }
     }
+    }   // pass
 }
 
 // ------------------------------------------------------------------------------------------------ gated linear recurrence
@@ -1115,8 +1121,8 @@ extern "C" int mi355_hy_attn_tiles(const float* q, int32_t ldq, float scale, con
     }
     const int gq = g.H / g.G, nwv = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;       // query heads of one key/value head per block
 #define HY_TILES(DKM_, NCBM_, NWV_)                                                                                                            \
-    hipLaunchKernelGGL((hy_attn_tiles_kernel<DKM_, NCBM_, NWV_>), dim3(tiles, g.H / NWV_), dim3(64 * NWV_), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, \
-                       sink, vfreq, pos, seq, block_table, tile_row0, tile_n, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out)
+    hipLaunchKernelGGL((hy_attn_tiles_kernel<DKM_, NCBM_, NWV_>), dim3((tiles + 1) / 2, g.H / NWV_), dim3(64 * NWV_), 0, (hipStream_t)stream, q, ldq, scale, g, chunk, \
+                       sink, vfreq, pos, seq, block_table, tile_row0, tile_n, tiles, (const bf16*)kcache, (const bf16*)vcache, (bf16*)out)
     if (g.dim <= 128 && g.vdim <= 128) { if (nwv == 4) HY_TILES(4, 8, 4); else if (nwv == 2) HY_TILES(4, 8, 2); else HY_TILES(4, 8, 1); }
     else                               { if (nwv == 4) HY_TILES(8, 16, 4); else if (nwv == 2) HY_TILES(8, 16, 2); else HY_TILES(8, 16, 1); }
 #undef HY_TILES
