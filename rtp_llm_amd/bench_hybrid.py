@@ -419,9 +419,9 @@ def kernel_table_pokepel(s, dev, prompt):
         x, a, b, gt = f32(T_, W), f32(T_, W), f32(T_, W), f32(T_, 2 * W)
         w1, w2 = bf(W), bf(W)
         t = timed_k(lambda: hops.residual_norm(x, a, b, 1.0, w1, None, 1e-6, gate=gt))
-        add("pokepel", "gated residual + norm (fp32 stream)", f"M={T_} W={W}", t, M_bytes(T_, W, 6, 1), 0, VALU_F32)
+        add("pokepel", "gated residual + norm (fp32 stream)", f"M={T_} W={W}", t, stream_bytes(T_, W, 6, 1), 0, VALU_F32)
         t = timed_k(lambda: hops.residual_norm(x, a, b, 0.3, w1, w2, 1e-5, weight_offset=1.0))
-        add("nufalorn", "residual + 2 norms (fp32 stream)", f"M={T_} W={W}", t, M_bytes(T_, W, 4, 2), 0, VALU_F32)
+        add("nufalorn", "residual + 2 norms (fp32 stream)", f"M={T_} W={W}", t, stream_bytes(T_, W, 4, 2), 0, VALU_F32)
     # recurrence: fixed decay (after the separate turn of q and k) against the gated-linear-attention scan
     d = hd // 2
     for T_, name in ((prompt, "prefill"), (8, "decode b=8")):
@@ -444,7 +444,7 @@ def kernel_table_pokepel(s, dev, prompt):
     return rows
 
 
-def M_bytes(T_, W, f32_streams, bf16_streams):
+def stream_bytes(T_, W, f32_streams, bf16_streams):
     return T_ * W * (4 * f32_streams + 2 * bf16_streams)
 
 

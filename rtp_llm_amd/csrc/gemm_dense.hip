@@ -7,6 +7,8 @@
 //   * tile kernel, fp32:  64 x 64 block tile, 4 x 4 register micro-tiles, true fp32 FMAs (no reduced-precision matrix mode);
 //   * skinny kernel, bf16, 2 <= M <= 16: one block per 16 outputs, its waves split K, MFMA fragments loaded straight from memory;
 //   * row kernel (M = 1; fp32 up to M = 16): a wave per output column streams its weight row once, 16-byte loads, wave reduction at the end.
+//   * grouped forms of the tile kernels (per-head weights over column slices, or rows sorted by expert with a gather and a tile list) and
+//     of the row kernel (the few rows of a decode step, each with its own expert's weight): mi355_dense_grouped.
 // Epilogues: bias, gated activation act(gate) * up (weight rows grouped [32 gate | 32 up], so one lane holds both), tanh soft cap.
 // Output is fp32 or the activation type.  A result row depends only on its own input row: the k order of the accumulation is fixed by
 // the kernel, never by M or by the row's place in the batch.

@@ -1,7 +1,9 @@
-// Kernels of the hybrid decoder family: layers x <- x + m * (mixer(norm1 x) + ffn(norm2 x)) over an fp32 residual stream, whose token mixer is
-// either paged attention (chunk-local causal mask, optional sink in the softmax denominator, unit-normed values that are rotated by their
-// position and turned back at the query's position) or a gated linear recurrence S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with
-// its state in fp32 slots (HGRN2 and gated-linear-attention parametrisations of a, k, q).
+// Kernels of the hybrid decoder family: layers x <- x + m * (g1 * mixer(norm1 x) + g2 * ffn(norm2 x)) over an fp32 residual stream (g: optional
+// per-channel sigmoid gates), whose token mixer is paged attention (chunk-local or plain causal mask, optional sink logit in the softmax
+// denominator, optionally unit-normed values that are rotated by their position and turned back at the query's position; or low-rank latent
+// attention over one cached row per token that serves as key and, with its leading channels, as value) or a linear recurrence
+// S_t = diag(a_t) S_(t-1) + k_t v_t^T, o_t = S_t^T q_t with its state in fp32 slots (HGRN2, gated-linear-attention and fixed-decay retention
+// parametrisations of a, k, q); feed-forward helpers: PolyNorm, and routing / sorting / weighted sum of a mixture of experts.
 //
 // One ragged batch of rows serves prefill portions and decode tokens alike: every row carries its position and the index of its
 // sequence; a sequence carries its block-table row, its state slot and the range of its rows.  What the model states as 32-bit is fp32
