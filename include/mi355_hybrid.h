@@ -39,7 +39,8 @@ int mi355_hy_head_norm(const float* o, int32_t rows, int32_t H, int32_t vdim, co
                        int32_t goff, void* out, int32_t act_dtype, mi355_stream_t stream);
 int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y, int32_t ldy,
                         int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs, int64_t ys, const int32_t* offs,
-                        const int32_t* gather, const int32_t* tiles, int32_t max_tiles, mi355_stream_t stream);
+                        const int32_t* gather, const int32_t* tiles, int32_t max_tiles, const float* egate, int32_t ldg, int32_t goff,
+                        mi355_stream_t stream);
 int mi355_hy_gated_residual_norm(float* x, const float* a, const float* b, const float* gate, int32_t ldg, float mult, const int32_t* rows, int32_t n,
                                  int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
                                  mi355_stream_t stream);
@@ -50,12 +51,12 @@ int mi355_hy_rotary(float* buf, int32_t ld, int32_t rows, int32_t off0, int32_t 
                     int32_t dim1, float scale1, int32_t rdims, int32_t layout, const float* freq, float mag, const int32_t* pos, mi355_stream_t stream);
 int mi355_hy_polynorm(const float* z, int32_t ld, int32_t rows, int32_t n, float ca, float cb, float cc, float ce, float eps, void* out, int32_t ldo,
                       int32_t act_dtype, mi355_stream_t stream);
-int mi355_hy_gate_mul(const float* o, int32_t rows, int32_t n, const float* gate, int32_t ldg, int32_t goff, void* out, int32_t act_dtype,
-                      mi355_stream_t stream);
 int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
                        mi355_stream_t stream);
 int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, int32_t E, int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles,
                        mi355_stream_t stream);
+int mi355_hy_moe_route_align(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                             int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, mi355_stream_t stream);
 int mi355_hy_moe_combine(const float* y, int32_t tokens, int32_t W, const int32_t* place_of, const float* wts, int32_t top, const float* extra, float* out,
                          mi355_stream_t stream);
 

@@ -34,6 +34,8 @@ struct DenseParams {
     int G;
     long long xs, ws, ys;
     const int32_t* offs; const int32_t* gather; const int32_t* tiles;
+    // y[row, col] is multiplied by sigmoid(egate[row * ldg + goff + col]) before it is stored (fp32 pre-activations; null: no gate)
+    const float* egate; int ldg, goff;
 };
 
 // first row and end of the rows of the block's tile in its group, and the group's operand bases
@@ -63,6 +65,7 @@ template <typename T> __device__ __forceinline__ float dn_ld(const T* p) { retur
 template <typename T>
 __device__ __forceinline__ void dn_store(const DenseParams& p, int row, int col, float v) {
     if (p.softcap > 0.f) v = p.softcap * tanhf(v / p.softcap);
+    if (p.egate) v *= 1.f / (1.f + expf(-p.egate[(size_t)row * p.ldg + p.goff + col]));
     if (p.out_f32) ((float*)p.y)[(size_t)row * p.ldy + col] = v;
     else           ((T*)p.y)[(size_t)row * p.ldy + col] = (T)v;
 }
@@ -477,7 +480,7 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
     p.x = x; p.w = w; p.bias = bias; p.y = y; p.M = M; p.N = N; p.K = K; p.ldx = ldx; p.ldy = ldy;
     p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = softcap;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
-    p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr; p.tiles = nullptr;
+    p.G = 1; p.xs = p.ws = p.ys = 0; p.offs = nullptr; p.gather = nullptr; p.tiles = nullptr; p.egate = nullptr; p.ldg = p.goff = 0;
     (void)es;
     hipStream_t st = (hipStream_t)stream;
     if (bf && M > 1 && M <= 16 && p.vec) {
@@ -512,10 +515,11 @@ extern "C" int mi355_dense_linear(const void* x, int32_t ldx, int32_t M, const v
 // sorted row r reads x row gather[r] (device, or null for r itself) and writes y row r (experts of a mixture: xs = ys = 0).  A row's result
 // depends on its own input and its group's weight only.  tiles (device, with offs; null: every group is given ceil(M / 64) row tiles, most of
 // them empty): {n, (group, first row) x n}, the 64-row tiles that hold rows, at most max_tiles of them (mi355_hy_moe_align writes the list).
+// egate (fp32 [M, ldg], or null): y[m, c] is multiplied by sigmoid(egate[m, goff + c]), c counted over the whole output row.
 extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, int32_t N, int32_t K, const void* bias, void* y,
                                    int32_t ldy, int32_t out_f32, int32_t gated, int32_t act, int32_t act_dtype, int32_t G, int64_t xs,
                                    int64_t ys, const int32_t* offs, const int32_t* gather, const int32_t* tiles, int32_t max_tiles,
-                                   mi355_stream_t stream) {
+                                   const float* egate, int32_t ldg, int32_t goff, mi355_stream_t stream) {
     MI355_CHECK_ARG(x && w && y && M > 0 && N > 0 && K > 0 && G > 0 && xs >= 0 && ys >= 0, "dense_grouped: M=%d N=%d K=%d G=%d", M, N, K, G);
     MI355_CHECK_ARG(ldx >= xs * (G - 1) + K, "dense_grouped: ldx=%d for %d groups of K=%d at step %lld", ldx, G, K, (long long)xs);
     MI355_CHECK_ARG(act_dtype == MI355_ACT_BF16 || act_dtype == MI355_ACT_F32, "dense_grouped: act_dtype=%d (bf16 or fp32)", act_dtype);
@@ -529,6 +533,8 @@ extern "C" int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const 
     p.gated = gated; p.act = act; p.out_f32 = bf ? out_f32 : 1; p.softcap = 0.f;
     p.vec = (K % 8 == 0) && (ldx % 8 == 0) && (xs % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
     p.G = G; p.xs = xs; p.ws = (long long)N * K; p.ys = ys; p.offs = offs; p.gather = gather; p.tiles = tiles;
+    p.egate = egate; p.ldg = ldg; p.goff = goff;
+    MI355_CHECK_ARG(!egate || (goff >= 0 && ldg >= goff + (offs ? 0 : ys * (G - 1)) + (gated ? N / 2 : N)), "dense_grouped: gate row stride %d", ldg);
     static_assert(TB_M == 64 && TF_M == 64, "the tile list is made of 64-row tiles");
     hipStream_t st = (hipStream_t)stream;
     const int gy = tiles ? max_tiles : (M + 63) / 64, gz = tiles ? 1 : G;

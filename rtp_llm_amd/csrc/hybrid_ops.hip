@@ -908,14 +908,6 @@ __global__ __launch_bounds__(256) void hy_polynorm_kernel(const float* z, int ld
     }
 }
 
-// out = (T)(o * sigmoid(gate)) elementwise: o fp32 [rows, n], gate fp32 [rows, ldg] from column goff
-template <typename T>
-__global__ __launch_bounds__(256) void hy_gate_mul_kernel(const float* o, int n, const float* gate, int ldg, int goff, T* out) {
-    const int r = blockIdx.x;
-    for (int c = threadIdx.x; c < n; c += 256)
-        out[(size_t)r * n + c] = (T)(o[(size_t)r * n + c] * hy_sigmoid(gate[(size_t)r * ldg + goff + c]));
-}
-
 // ------------------------------------------------------------------------------------------------ mixture of experts: routing, sorting by expert, weighted sum
 // One wave per token: softmax over the E router logits (fp32); experts come in `groups` runs of E / groups neighbours, a group scores as its
 // best expert and only the `keep` best groups stay eligible; the `top` eligible experts with the largest scores are chosen, ties to the lower
@@ -929,59 +921,62 @@ __device__ __forceinline__ void hy_wave_argmax(float& v, int& i) {
     }
 }
 
-__global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld, int E, int groups, int keep, int top, int32_t* ids, float* wts) {
-    extern __shared__ float hy_rs[];            // scores [E], group best [groups]
-    float* sc = hy_rs;
-    float* gb = hy_rs + E;
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const float* zr = z + (size_t)t * ld;
+// The routing of one token by one wave; sc [E] and gb [groups] are the wave's scratch in LDS.  Every thread of the block calls it the same
+// number of times (it holds block barriers); a wave without a token passes active = false.
+__device__ __forceinline__ void hy_route_token(bool active, const float* zr, float* sc, float* gb, int E, int groups, int keep, int top, int32_t* ids,
+                                               float* wts, int lane) {
     float m = -INFINITY;
-    for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
+    if (active) for (int e = lane; e < E; e += 64) m = fmaxf(m, zr[e]);
     m = hy_wave_max(m);
     float sum = 0.f;
-    for (int e = lane; e < E; e += 64) { const float x = expf(zr[e] - m); sc[e] = x; sum += x; }
+    if (active) for (int e = lane; e < E; e += 64) { const float x = expf(zr[e] - m); sc[e] = x; sum += x; }
     sum = hy_wave_sum(sum);
-    for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
+    if (active) for (int e = lane; e < E; e += 64) sc[e] = sc[e] / sum;
     __syncthreads();
     const int per = E / groups;
     if (groups > 1 && keep < groups) {
-        for (int g = lane; g < groups; g += 64) {
-            float b = -1.f;
-            for (int j = 0; j < per; ++j) b = fmaxf(b, sc[g * per + j]);
-            gb[g] = b;
-        }
+        if (active)
+            for (int g = lane; g < groups; g += 64) {
+                float b = -1.f;
+                for (int j = 0; j < per; ++j) b = fmaxf(b, sc[g * per + j]);
+                gb[g] = b;
+            }
         __syncthreads();
         for (int k = 0; k < keep; ++k) {          // the kept groups get a best score of 2 (above any probability), the others stay below
             float bv = -2.f; int bi = 0x7fffffff;
-            for (int g = lane; g < groups; g += 64) { const float v = gb[g]; if (v <= 1.5f && (v > bv || (v == bv && g < bi))) { bv = v; bi = g; } }
+            if (active) for (int g = lane; g < groups; g += 64) { const float v = gb[g]; if (v <= 1.5f && (v > bv || (v == bv && g < bi))) { bv = v; bi = g; } }
             hy_wave_argmax(bv, bi);
-            if (lane == 0) gb[bi] = 2.f;
+            if (active && lane == 0) gb[bi] = 2.f;
             __syncthreads();
         }
     } else {
-        for (int g = lane; g < groups; g += 64) gb[g] = 2.f;
+        if (active) for (int g = lane; g < groups; g += 64) gb[g] = 2.f;
         __syncthreads();
     }
     for (int k = 0; k < top; ++k) {
         float bv = -2.f; int bi = 0x7fffffff;
-        for (int e = lane; e < E; e += 64) {
-            const float v = sc[e];
-            if (v >= 0.f && gb[e / per] > 1.5f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
-        }
+        if (active)
+            for (int e = lane; e < E; e += 64) {
+                const float v = sc[e];
+                if (v >= 0.f && gb[e / per] > 1.5f && (v > bv || (v == bv && e < bi))) { bv = v; bi = e; }
+            }
         hy_wave_argmax(bv, bi);
-        if (lane == 0) { ids[(size_t)t * top + k] = bi; wts[(size_t)t * top + k] = bv; sc[bi] = -1.f; }     // taken
+        if (active && lane == 0) { ids[k] = bi; wts[k] = bv; sc[bi] = -1.f; }     // taken
         __syncthreads();
     }
+}
+
+__global__ __launch_bounds__(64) void hy_moe_route_kernel(const float* z, int ld, int E, int groups, int keep, int top, int32_t* ids, float* wts) {
+    extern __shared__ float hy_rs[];            // scores [E], group best [groups]
+    const int t = blockIdx.x;
+    hy_route_token(true, z + (size_t)t * ld, hy_rs, hy_rs + E, E, groups, keep, top, ids + (size_t)t * top, wts + (size_t)t * top, threadIdx.x);
 }
 
 // Counting sort of the n = tokens * top (token, choice) pairs by expert, one block: offs [E + 1], src_row[sorted place] = token,
 // place_of[pair] = sorted place, tiles = {count, (expert, first row) x count}: the 64-row tiles of the sorted list that hold rows.  The order
 // inside an expert is arbitrary (rows are independent of each other).
-__global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, int n, int top, int E, int32_t* offs, int32_t* src_row, int32_t* place_of,
-                                                            int32_t* tiles) {
-    extern __shared__ int hy_cnt[];             // counts [E], cursors [E]
-    int* cnt = hy_cnt;
-    int* cur = hy_cnt + E;
+__device__ __forceinline__ void hy_align_pairs(const int32_t* ids, int n, int top, int E, int* cnt, int* cur, int32_t* offs, int32_t* src_row,
+                                               int32_t* place_of, int32_t* tiles) {
     for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
     for (int i = threadIdx.x; i < n; i += blockDim.x) atomicAdd(&cnt[ids[i]], 1);
@@ -1001,6 +996,30 @@ __global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, 
         src_row[at] = i / top;
         place_of[i] = at;
     }
+}
+
+__global__ __launch_bounds__(1024) void hy_moe_align_kernel(const int32_t* ids, int n, int top, int E, int32_t* offs, int32_t* src_row, int32_t* place_of,
+                                                            int32_t* tiles) {
+    extern __shared__ int hy_cnt[];             // counts [E], cursors [E]
+    hy_align_pairs(ids, n, top, E, hy_cnt, hy_cnt + E, offs, src_row, place_of, tiles);
+}
+
+// Routing and sorting of a few tokens (a decode step) in ONE block: its sixteen waves route a token each per trip, then the block sorts the pairs.
+__global__ __launch_bounds__(1024) void hy_moe_route_align_kernel(const float* z, int ld, int T, int E, int groups, int keep, int top, int32_t* ids, float* wts,
+                                                                  int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles) {
+    extern __shared__ float hy_ra[];            // per wave: scores [E], group best [groups]; then counts [E], cursors [E]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float* sc = hy_ra + (size_t)wave * (E + groups);
+    for (int t0 = 0; t0 < T; t0 += 16) {
+        const int t = t0 + wave;
+        const bool active = t < T;
+        hy_route_token(active, z + (size_t)(active ? t : 0) * ld, sc, sc + E, E, groups, keep, top, ids + (size_t)(active ? t : 0) * top,
+                       wts + (size_t)(active ? t : 0) * top, lane);
+    }
+    __threadfence_block();
+    __syncthreads();
+    int* cnt = (int*)(hy_ra + (size_t)16 * (E + groups));
+    hy_align_pairs(ids, T * top, top, E, cnt, cnt + E, offs, src_row, place_of, tiles);
 }
 
 // out[t] = sum_k wts[t, k] * y[place_of[t * top + k]] (+ extra[t]): fp32 [tokens, W], the choices added in order k = 0 .. top - 1
@@ -1206,14 +1225,6 @@ extern "C" int mi355_hy_polynorm(const float* z, int32_t ld, int32_t rows, int32
     return MI355_OK;
 }
 
-extern "C" int mi355_hy_gate_mul(const float* o, int32_t rows, int32_t n, const float* gate, int32_t ldg, int32_t goff, void* out, int32_t act_dtype,
-                                 mi355_stream_t stream) {
-    MI355_CHECK_ARG(o && gate && out && rows > 0 && n > 0 && goff >= 0 && ldg >= goff + n, "hy_gate_mul: rows=%d n=%d", rows, n);
-    HY_DISPATCH(act_dtype, hipLaunchKernelGGL(hy_gate_mul_kernel<T>, dim3(rows), dim3(256), 0, (hipStream_t)stream, o, n, gate, ldg, goff, (T*)out));
-    MI355_CHECK_LAUNCH("hy_gate_mul_kernel");
-    return MI355_OK;
-}
-
 // z fp32 [tokens, ld] router logits -> ids int32 [tokens, top], wts fp32 [tokens, top]
 extern "C" int mi355_hy_moe_route(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
                                   mi355_stream_t stream) {
@@ -1232,6 +1243,22 @@ extern "C" int mi355_hy_moe_align(const int32_t* ids, int32_t n, int32_t top, in
     MI355_CHECK_ARG(ids && offs && src_row && place_of && tiles && n > 0 && top > 0 && E > 0 && (size_t)E * 8 <= 48 * 1024, "hy_moe_align: n=%d experts=%d", n, E);
     hipLaunchKernelGGL(hy_moe_align_kernel, dim3(1), dim3(1024), (size_t)E * 8, (hipStream_t)stream, ids, n, top, E, offs, src_row, place_of, tiles);
     MI355_CHECK_LAUNCH("hy_moe_align_kernel");
+    return MI355_OK;
+}
+
+// Both in one launch for a few tokens (tokens <= 64 and the scratch of sixteen waves fits: MI355_ERR_UNSUPPORTED otherwise).
+extern "C" int mi355_hy_moe_route_align(const float* z, int32_t ld, int32_t tokens, int32_t E, int32_t groups, int32_t keep, int32_t top, int32_t* ids, float* wts,
+                                        int32_t* offs, int32_t* src_row, int32_t* place_of, int32_t* tiles, mi355_stream_t stream) {
+    MI355_CHECK_ARG(z && ids && wts && offs && src_row && place_of && tiles && tokens > 0 && E > 0 && ld >= E, "hy_moe_route_align: tokens=%d experts=%d", tokens, E);
+    MI355_CHECK_ARG(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= (E / groups) * keep, "hy_moe_route_align: %d experts in %d groups, keep %d, top %d",
+                    E, groups, keep, top);
+    const size_t lds = (size_t)16 * (E + groups) * 4 + (size_t)E * 8;
+    if (tokens > 64 || lds > 48 * 1024) {
+        mi355_set_error("hy_moe_route_align: %d tokens, %d experts: use the two launches", tokens, E);
+        return MI355_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(hy_moe_route_align_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream, z, ld, tokens, E, groups, keep, top, ids, wts, offs, src_row, place_of, tiles);
+    MI355_CHECK_LAUNCH("hy_moe_route_align_kernel");
     return MI355_OK;
 }
 

@@ -236,8 +236,9 @@ def head_norm(o: torch.Tensor, heads: int, vdim: int, w: Optional[torch.Tensor],
 
 def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: int = 0, offs: Optional[torch.Tensor] = None,
                   gather: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None, rows: Optional[int] = None, out_dtype: Optional[torch.dtype] = None, gated: bool = False,
-                  act: int = ACT_NONE, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One launch of G = w.shape[0] linears with the weights w [G, N, K].
+                  act: int = ACT_NONE, out: Optional[torch.Tensor] = None, mul_sigmoid: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One launch of G = w.shape[0] linears with the weights w [G, N, K].  mul_sigmoid: fp32 [M, width of the output] pre-activations (a column
+    slice of a wider buffer is fine); every output is multiplied by the sigmoid of its entry before it is stored.
     Without offs every group takes all rows of x, reads its K inputs from column g * x_step and writes its outputs from column g * y_step
     (per-head projections).  With offs (int32 [G + 1] on the device) the `rows` rows of the output are sorted by group, group g owns rows
     offs[g] .. offs[g + 1] - 1, and sorted row r reads x[gather[r]] (x[r] without gather): the experts of a mixture.  tiles: the list of
@@ -268,10 +269,17 @@ def dense_grouped(x: torch.Tensor, w: torch.Tensor, *, x_step: int = 0, y_step: 
         raise _C.Mi355Error(f"dense_grouped: offs has {offs.numel()} entries for {G} groups")
     if gather is not None and gather.numel() < M:
         raise _C.Mi355Error(f"dense_grouped: gather has {gather.numel()} entries for {M} rows")
+    ldg = 0
+    if mul_sigmoid is not None:
+        _dev(mul_sigmoid, torch.float32, "dense_grouped.mul_sigmoid")
+        ldg = _rows(mul_sigmoid, "dense_grouped.mul_sigmoid")
+        if mul_sigmoid.shape != (M, width):
+            raise _C.Mi355Error(f"dense_grouped: gate {tuple(mul_sigmoid.shape)} for outputs [{M}, {width}]")
     if M:
         _C.check_hybrid(_C.hybrid_lib().mi355_dense_grouped(x.data_ptr(), ldx, M, w.data_ptr(), N, K, None, out.data_ptr(), _rows(out, "dense_grouped.out"),
                                                             1 if od == torch.float32 else 0, 1 if gated else 0, act, act_code(w.dtype), G, x_step, y_step,
-                                                            _p(offs), _p(gather), _p(tiles), 0 if tiles is None else (tiles.numel() - 1) // 2, _stream()),
+                                                            _p(offs), _p(gather), _p(tiles), 0 if tiles is None else (tiles.numel() - 1) // 2, _p(mul_sigmoid), ldg, 0,
+                                                            _stream()),
                         "dense_grouped")
     return out
 
@@ -324,19 +332,6 @@ def polynorm(z: torch.Tensor, coef, eps: float, dtype: torch.dtype) -> torch.Ten
     return out
 
 
-def gate_mul(o: torch.Tensor, gate: torch.Tensor, goff: int, dtype: torch.dtype) -> torch.Tensor:
-    """o * sigmoid(gate[:, goff : goff + n]) for fp32 o [T, n] -> `dtype`."""
-    _dev(o, torch.float32, "gate_mul.o"); _dev(gate, torch.float32, "gate_mul.gate")
-    if not o.is_contiguous():
-        raise _C.Mi355Error("gate_mul: o must be contiguous")
-    T, n = o.shape
-    out = torch.empty(T, n, dtype=dtype, device=o.device)
-    if T:
-        _C.check_hybrid(_C.hybrid_lib().mi355_hy_gate_mul(o.data_ptr(), T, n, gate.data_ptr(), _rows(gate, "gate_mul.gate"), goff, out.data_ptr(),
-                                                          act_code(dtype), _stream()), "hy_gate_mul")
-    return out
-
-
 def moe_route(z: torch.Tensor, groups: int, keep: int, top: int):
     """Router logits fp32 [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top]): softmax scores, only experts of the `keep` best of
     `groups` runs of neighbouring experts (a run scores as its best member) are eligible, the `top` best eligible are chosen."""
@@ -364,6 +359,24 @@ def moe_align(ids: torch.Tensor, experts: int):
         _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_align(ids.data_ptr(), T * top, top, experts, offs.data_ptr(), src.data_ptr(), place.data_ptr(),
                                                            tiles.data_ptr(), _stream()), "hy_moe_align")
     return offs, src, place, tiles
+
+
+def moe_route_sorted(z: torch.Tensor, experts: int, groups: int, keep: int, top: int):
+    """moe_route followed by moe_align -> (ids, wts, offs, src_row, place_of, tiles); a few tokens (a decode step) take one launch for both."""
+    _dev(z, torch.float32, "moe_route_sorted.z")
+    T = z.shape[0]
+    if z.shape[1] != experts:
+        raise _C.Mi355Error(f"moe_route_sorted: logits {tuple(z.shape)} for {experts} experts")
+    if not 0 < T <= 64 or 16 * (experts + groups) * 4 + experts * 8 > 48 * 1024:
+        ids, wts = moe_route(z, groups, keep, top)
+        return (ids, wts) + moe_align(ids, experts)
+    dev = z.device
+    ids, wts = torch.empty(T, top, dtype=torch.int32, device=dev), torch.empty(T, top, dtype=torch.float32, device=dev)
+    offs, src, place = torch.empty(experts + 1, dtype=torch.int32, device=dev), torch.empty(T * top, dtype=torch.int32, device=dev), torch.empty(T * top, dtype=torch.int32, device=dev)
+    tiles = torch.empty(1 + 2 * (T * top // 64 + experts), dtype=torch.int32, device=dev)
+    _C.check_hybrid(_C.hybrid_lib().mi355_hy_moe_route_align(z.data_ptr(), _rows(z, "moe_route_sorted.z"), T, experts, groups, keep, top, ids.data_ptr(), wts.data_ptr(),
+                                                             offs.data_ptr(), src.data_ptr(), place.data_ptr(), tiles.data_ptr(), _stream()), "hy_moe_route_align")
+    return ids, wts, offs, src, place, tiles
 
 
 def moe_combine(y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -271,8 +271,8 @@ class LatentAttention:
             ol = hops.attn_tiles(qabs, s.scale, ageom, 0, self.sink, None, batch.pos, batch.seq, batch.block_table, batch.tile_row0, batch.tile_n, kc, kc, H, R)
         else:
             ol = hops.attn_rows(qabs, s.scale, ageom, 0, self.sink, None, batch.pos, batch.seq, batch.block_table, kc, kc, H, R)
-        o = hops.dense_grouped(ol, self.w_uv, x_step=R, y_step=s.vdim, out_dtype=torch.float32)
-        o = hops.gate_mul(o, proj, self.goff, self.act) if s.out_gate else o.to(self.act)
+        # value up-projection per head; the output gate sigmoid(W_g h) is applied in its epilogue
+        o = hops.dense_grouped(ol, self.w_uv, x_step=R, y_step=s.vdim, mul_sigmoid=proj[:, self.goff:self.goff + H * s.vdim] if s.out_gate else None)
         return hops.dense_linear(o, self.w_o, out_dtype=torch.float32)
 
 
@@ -370,8 +370,7 @@ class RoutedExperts:
         r = self.router
         if logits is None:
             logits = hops.dense_linear(h, self.w_router, out_dtype=torch.float32)
-        ids, wts = hops.moe_route(logits, r.groups, r.keep, r.top)
-        offs, src, place, tiles = hops.moe_align(ids, r.experts)
+        ids, wts, offs, src, place, tiles = hops.moe_route_sorted(logits, r.experts, r.groups, r.keep, r.top)
         n = ids.numel()
         a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=self.act)
         y = hops.dense_grouped(a, self.w_down, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32)

@@ -54,6 +54,10 @@ def test_grouped_linear_heads_and_sorted_rows():
             y = hops.dense_grouped(x, w, x_step=K, y_step=N + 3, out_dtype=torch.float32)
             for j in range(G):
                 close(y[:, j * (N + 3):j * (N + 3) + N], (x[:, j * K:(j + 1) * K].double() @ w[j].double().T).cpu(), tol)
+            gate = torch.randn(M, G * N + 5, device=DEV, generator=g)                # outputs times the sigmoid of a slice of a wider buffer
+            y = hops.dense_grouped(x, w, x_step=K, y_step=N, out_dtype=torch.float32, mul_sigmoid=gate[:, 2:2 + G * N])
+            ref = torch.cat([x[:, j * K:(j + 1) * K].double() @ w[j].double().T for j in range(G)], 1) * torch.sigmoid(gate[:, 2:2 + G * N].double())
+            close(y, ref.cpu(), tol)
         # rows sorted by group with a gather on the input, empty groups, groups larger than a tile; gated epilogue
         E, K, ff, T = 6, 40, 32, 90
         for counts in ([0, 75, 1, 0, 130, 3], [0, 2, 1, 0, 5, 3], [0, 0, 0, 1, 0, 0]):      # prompt-sized, and the few rows of a decode step
@@ -110,20 +114,27 @@ def test_polynorm_activation():
 @pytest.mark.parametrize("E,groups,keep,top", [(8, 4, 2, 2), (12, 3, 1, 3), (6, 1, 1, 1), (64, 8, 4, 6), (130, 2, 2, 5), (9, 9, 3, 3)])
 def test_router_choices_and_weights(E, groups, keep, top):
     from rtp_llm_amd import hybrid_ops as hops
-    z = torch.randn(50, E, generator=torch.Generator().manual_seed(E)) * 3
+    z = torch.randn(100, E, generator=torch.Generator().manual_seed(E)) * 3
     ids, wts = hops.moe_route(z.to(DEV), groups, keep, top)
     router = {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}}
     want_ids, want_w = O.route(z.double(), {"r.router": torch.eye(E, dtype=torch.float64)}, "r.", router)       # identity router: logits = z
     assert torch.equal(ids.cpu().long(), want_ids)
     close(wts, want_w, 1e-6)
-    offs, src, place, tiles = hops.moe_align(ids, E)
-    offs, src, place, tiles = offs.cpu(), src.cpu(), place.cpu(), tiles.cpu().tolist()
-    want_tiles = [(e, m) for e in range(E) for m in range(int(offs[e]), int(offs[e + 1]), 64)]
-    assert tiles[0] == len(want_tiles) and list(zip(tiles[1:1 + 2 * tiles[0]:2], tiles[2:2 + 2 * tiles[0]:2])) == want_tiles
-    flat = ids.cpu().flatten()
-    assert offs[0] == 0 and offs[-1] == flat.numel() and sorted(place.tolist()) == list(range(flat.numel()))
-    for i, e in enumerate(flat.tolist()):
-        assert offs[e] <= place[i] < offs[e + 1] and src[place[i]] == i // top
+    def check_sort(ids, offs, src, place, tiles):
+        offs, src, place, tiles = offs.cpu(), src.cpu(), place.cpu(), tiles.cpu().tolist()
+        want_tiles = [(e, m) for e in range(E) for m in range(int(offs[e]), int(offs[e + 1]), 64)]
+        assert tiles[0] == len(want_tiles) and list(zip(tiles[1:1 + 2 * tiles[0]:2], tiles[2:2 + 2 * tiles[0]:2])) == want_tiles
+        flat = ids.cpu().flatten()
+        assert offs[0] == 0 and offs[-1] == flat.numel() and sorted(place.tolist()) == list(range(flat.numel()))
+        for i, e in enumerate(flat.tolist()):
+            assert offs[e] <= place[i] < offs[e + 1] and src[place[i]] == i // top
+
+    check_sort(ids, *hops.moe_align(ids, E))
+    for T in (1, 17, 50, 100):                                   # up to 64 tokens: routing and sorting in one launch; more: the two launches
+        got = hops.moe_route_sorted(z[:T].to(DEV), E, groups, keep, top)
+        assert torch.equal(got[0].cpu().long(), want_ids[:T])
+        close(got[1], want_w[:T], 1e-6)
+        check_sort(got[0], *got[2:])
 
 
 # ------------------------------------------------------------------------------------------------ mechanisms alone
