@@ -42,8 +42,8 @@ int mi355_dense_grouped(const void* x, int32_t ldx, int32_t M, const void* w, in
                         const int32_t* gather, const int32_t* tiles, int32_t max_tiles, const float* egate, int32_t ldg, int32_t goff,
                         mi355_stream_t stream);
 int mi355_hy_gated_residual_norm(float* x, const float* a, const float* b, const float* gate, int32_t ldg, float mult, const int32_t* rows, int32_t n,
-                                 int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
-                                 mi355_stream_t stream);
+                                 int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, const float* moe_y,
+                                 const int32_t* moe_place, const float* moe_wts, int32_t moe_top, int32_t act_dtype, mi355_stream_t stream);
 int mi355_hy_latent_prep(const float* proj, int32_t ld, int32_t doff, const int32_t* geom, const float* freq, float mag, const void* cw, float eps,
                          const int32_t* pos, const int32_t* seq, const int32_t* block_table, int32_t rows, void* qn, float* qabs, void* cache,
                          int32_t act_dtype, mi355_stream_t stream);

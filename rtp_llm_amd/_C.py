@@ -174,7 +174,7 @@ HYBRID_SIGNATURES = {
     "mi355_hy_scan": (i32, [i32, vp, i32, i32, i32, i32, vp, i32, vp, vp, f32, f32, i32, i32, i32, vp, vp, vp, i32, vp, vp, i32, vp]),
     "mi355_hy_head_norm": (i32, [vp, i32, i32, i32, vp, f32, vp, i32, i32, vp, i32, vp]),
     "mi355_dense_grouped": (i32, [vp, i32, i32, vp, i32, i32, vp, vp, i32, i32, i32, i32, i32, i32, C.c_int64, C.c_int64, vp, vp, vp, i32, vp, i32, i32, vp]),
-    "mi355_hy_gated_residual_norm": (i32, [vp, vp, vp, vp, i32, f32, vp, i32, i32, vp, vp, f32, f32, vp, vp, i32, vp]),
+    "mi355_hy_gated_residual_norm": (i32, [vp, vp, vp, vp, i32, f32, vp, i32, i32, vp, vp, f32, f32, vp, vp, vp, vp, vp, i32, i32, vp]),
     "mi355_hy_latent_prep": (i32, [vp, i32, i32, ip, vp, f32, vp, f32, vp, vp, vp, i32, vp, vp, vp, i32, vp]),
     "mi355_hy_rotary": (i32, [vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, f32, i32, i32, vp, f32, vp, vp]),
     "mi355_hy_polynorm": (i32, [vp, i32, i32, i32, f32, f32, f32, f32, f32, vp, i32, i32, vp]),

@@ -79,9 +79,12 @@ template <> __device__ __forceinline__ void hy_store4<bf16>(bf16* p, const float
 
 // x[src] <- x[src] + mult * (ga * a[src] + gb * b[src]) (written back unless rows are gathered), then h1 = norm(x) * (off + w1), h2 likewise.
 // gate null: ga = gb = 1; else ga = sigmoid(gate[src, c]) and gb = sigmoid(gate[src, W + c]) (fp32 pre-activations, row stride ldg).
+// ms.y non-null: the second branch is a mixture's weighted sum formed here, b[src] (if any) + sum_k ms.wts[src, k] * ms.y[ms.place[src, k]].
 // VEC: W % 4 == 0, four channels per thread and trip (16-byte accesses on the fp32 stream).
+struct MoeSum { const float* y; const int32_t* place; const float* wts; int top; };
+
 template <typename T, bool VEC>
-__global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, const float* gate, int ldg, float mult,
+__global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const float* a, const float* b, MoeSum ms, const float* gate, int ldg, float mult,
                                                                const int32_t* rows, const T* w1, const T* w2, float off, float eps, int W, T* h1, T* h2) {
     extern __shared__ __attribute__((aligned(16))) float hy_xs[];
     __shared__ float red[4];
@@ -93,15 +96,29 @@ __global__ __launch_bounds__(256) void hy_residual_norm_kernel(float* x, const f
         float v[4], ya[4] = {0.f, 0.f, 0.f, 0.f}, yb[4] = {0.f, 0.f, 0.f, 0.f};
         if (VEC) { hy_load4<float>(x + i, v); if (a) hy_load4<float>(a + i, ya); if (b) hy_load4<float>(b + i, yb); }
         else     { v[0] = x[i]; if (a) ya[0] = a[i]; if (b) yb[0] = b[i]; }
-        if (gate && (a || b)) {
+        const bool has_b = b || ms.y;
+        if (ms.y) {         // the chosen experts' outputs in choice order, then the shared expert's
+            float sum[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < ms.top; ++k) {
+                const float wk = ms.wts[(size_t)src * ms.top + k];
+                const float* yr = ms.y + (size_t)ms.place[(size_t)src * ms.top + k] * W + c;
+                float t[4] = {0.f, 0.f, 0.f, 0.f};
+                if (VEC) hy_load4<float>(yr, t); else t[0] = yr[0];
+#pragma unroll
+                for (int e = 0; e < V; ++e) sum[e] = __builtin_fmaf(wk, t[e], sum[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < V; ++e) yb[e] = sum[e] + yb[e];
+        }
+        if (gate && (a || has_b)) {
             float ga[4] = {0.f, 0.f, 0.f, 0.f}, gb[4] = {0.f, 0.f, 0.f, 0.f};
             const float* gp = gate + (size_t)src * ldg + c;
-            if (VEC) { if (a) hy_load4<float>(gp, ga); if (b) hy_load4<float>(gp + W, gb); }
-            else     { if (a) ga[0] = gp[0]; if (b) gb[0] = gp[W]; }
+            if (VEC) { if (a) hy_load4<float>(gp, ga); if (has_b) hy_load4<float>(gp + W, gb); }
+            else     { if (a) ga[0] = gp[0]; if (has_b) gb[0] = gp[W]; }
 #pragma unroll
             for (int e = 0; e < V; ++e) { ya[e] *= hy_sigmoid(ga[e]); yb[e] *= hy_sigmoid(gb[e]); }
         }
-        if (a || b) {
+        if (a || has_b) {
 #pragma unroll
             for (int e = 0; e < V; ++e) v[e] = v[e] + mult * (ya[e] + yb[e]);
             if (!rows) { if (VEC) hy_store4<float>(x + i, v); else x[i] = v[0]; }
@@ -1064,18 +1081,23 @@ extern "C" int mi355_hy_embed(const int32_t* ids, int32_t rows, const void* tabl
 // x [*, W] fp32 stream; a, b [*, W] fp32 branch outputs (either may be null); rows: null, or `n` source rows to gather (x is then read only).
 // h1 / h2 [n, W] of act_dtype: x / rms(x) * (weight_offset + w).  w2 / h2 may be null.
 // gate: null, or fp32 [*, ldg] pre-activations of per-channel branch gates: a is scaled by sigmoid(gate[:, 0:W]), b by sigmoid(gate[:, W:2W]).
+// moe_y non-null: the second branch is b (may be null) + sum_k moe_wts[r, k] * moe_y[moe_place[r, k]] (fp32 [pairs, W], int32 [*, top], fp32 [*, top]):
+// the weighted sum of a mixture's chosen experts, formed here instead of by mi355_hy_moe_combine.
 extern "C" int mi355_hy_gated_residual_norm(float* x, const float* a, const float* b, const float* gate, int32_t ldg, float mult, const int32_t* rows,
                                             int32_t n, int32_t W, const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2,
-                                            int32_t act_dtype, mi355_stream_t stream) {
+                                            const float* moe_y, const int32_t* moe_place, const float* moe_wts, int32_t moe_top, int32_t act_dtype,
+                                            mi355_stream_t stream) {
+    MI355_CHECK_ARG(!moe_y || (moe_place && moe_wts && moe_top > 0), "hy_residual_norm: a mixture's sum needs its places and weights");
+    const MoeSum ms{moe_y, moe_place, moe_wts, moe_top};
     MI355_CHECK_ARG(x && n > 0 && W > 0 && (!h1 || w1) && (!h2 || w2), "hy_residual_norm: n=%d W=%d", n, W);
     MI355_CHECK_ARG((size_t)W * 4 <= 64 * 1024, "hy_residual_norm: W=%d too wide for one block", W);
     MI355_CHECK_ARG(!gate || ldg >= 2 * W, "hy_residual_norm: gate row stride %d for two gates of %d", ldg, W);
     auto al = [](const void* p_) { return ((uintptr_t)p_ & 15) == 0; };
-    if (W % 4 == 0 && ldg % 4 == 0 && al(x) && al(a) && al(b) && al(gate) && al(w1) && al(w2) && al(h1) && al(h2))
-        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, gate, ldg,
+    if (W % 4 == 0 && ldg % 4 == 0 && al(x) && al(a) && al(b) && al(gate) && al(w1) && al(w2) && al(h1) && al(h2) && al(moe_y))
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, true>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, ms, gate, ldg,
                                                   mult, rows, (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
     else
-        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, gate, ldg,
+        HY_DISPATCH(act_dtype, hipLaunchKernelGGL((hy_residual_norm_kernel<T, false>), dim3(n), dim3(256), (size_t)W * 4, (hipStream_t)stream, x, a, b, ms, gate, ldg,
                                                   mult, rows, (const T*)w1, (const T*)w2, weight_offset, eps, W, (T*)h1, (T*)h2));
     MI355_CHECK_LAUNCH("hy_residual_norm_kernel");
     return MI355_OK;
@@ -1084,7 +1106,7 @@ extern "C" int mi355_hy_gated_residual_norm(float* x, const float* a, const floa
 extern "C" int mi355_hy_residual_norm(float* x, const float* a, const float* b, float mult, const int32_t* rows, int32_t n, int32_t W,
                                       const void* w1, const void* w2, float weight_offset, float eps, void* h1, void* h2, int32_t act_dtype,
                                       mi355_stream_t stream) {
-    return mi355_hy_gated_residual_norm(x, a, b, nullptr, 0, mult, rows, n, W, w1, w2, weight_offset, eps, h1, h2, act_dtype, stream);
+    return mi355_hy_gated_residual_norm(x, a, b, nullptr, 0, mult, rows, n, W, w1, w2, weight_offset, eps, h1, h2, nullptr, nullptr, nullptr, 0, act_dtype, stream);
 }
 
 // geom: {H, G, dim, vdim, rot_dims, rot_layout, v_layout, page, max_blocks, num_pages}.  qkv fp32 [rows, ld]: q heads at column 0 (rotated in

@@ -236,7 +236,7 @@ class HybridModel:
             if mlp is None:
                 b = None
             elif g is not None and isinstance(mlp, RoutedExperts):
-                b = mlp.forward(h2, g[:, 2 * cfg.width: 2 * cfg.width + L.router.experts])
+                b = mlp.forward(h2, g[:, 2 * cfg.width: 2 * cfg.width + L.router.experts], defer=True)   # summed by the next residual kernel
             else:
                 b = mlp.forward(h2)
         if collect is not None:

@@ -102,7 +102,15 @@ def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.Tensor], mult: float, w1: torch.Tensor,
+class MoeSum:
+    """A mixture's weighted sum still to be formed: sum_k wts[t, k] * y[place_of[t, k]] (+ extra[t]).  residual_norm takes it as a branch and
+    forms it while it updates the stream; moe_combine forms it on its own."""
+
+    def __init__(self, y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None):
+        self.y, self.place_of, self.wts, self.extra = y, place_of, wts, extra
+
+
+def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b, mult: float, w1: torch.Tensor,
                   w2: Optional[torch.Tensor], eps: float, *, weight_offset: float = 0.0, rows: Optional[torch.Tensor] = None,
                   gate: Optional[torch.Tensor] = None):
     """x <- x + mult * (a + b) on the fp32 stream (in place; skipped for absent branches, and x is only read when `rows` gathers), then
@@ -111,6 +119,12 @@ def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.
     _dev(x, torch.float32, "residual_norm.x")
     W = x.shape[1]
     n = x.shape[0] if rows is None else rows.numel()
+    ms = None
+    if isinstance(b, MoeSum):                 # b: a tensor, or the parts of a mixture's sum
+        ms, b = b, b.extra
+        _dev(ms.y, torch.float32, "residual_norm.moe.y"); _dev(ms.wts, torch.float32, "residual_norm.moe.wts"); _dev(ms.place_of, torch.int32, "residual_norm.moe.place")
+        if ms.wts.shape[0] != x.shape[0] or ms.y.shape != (ms.wts.numel(), W) or ms.place_of.numel() != ms.wts.numel() or not (ms.y.is_contiguous() and ms.wts.is_contiguous()):
+            raise _C.Mi355Error(f"residual_norm: mixture sum y {tuple(ms.y.shape)} wts {tuple(ms.wts.shape)} against the stream {tuple(x.shape)}")
     for t, nm in ((a, "a"), (b, "b")):
         if t is not None:
             _dev(t, torch.float32, "residual_norm." + nm)
@@ -131,7 +145,8 @@ def residual_norm(x: torch.Tensor, a: Optional[torch.Tensor], b: Optional[torch.
     if n:
         _C.check_hybrid(_C.hybrid_lib().mi355_hy_gated_residual_norm(x.data_ptr(), _p(a), _p(b), _p(gate), ldg, float(mult), _p(rows), n, W,
                                                                      w1.data_ptr(), _p(w2), float(weight_offset), float(eps), h1.data_ptr(), _p(h2),
-                                                                     act_code(w1.dtype), _stream()), "hy_residual_norm")
+                                                                     _p(ms.y) if ms else None, _p(ms.place_of) if ms else None, _p(ms.wts) if ms else None,
+                                                                     ms.wts.shape[1] if ms else 0, act_code(w1.dtype), _stream()), "hy_residual_norm")
     return h1, h2
 
 
@@ -379,8 +394,10 @@ def moe_route_sorted(z: torch.Tensor, experts: int, groups: int, keep: int, top:
     return ids, wts, offs, src, place, tiles
 
 
-def moe_combine(y: torch.Tensor, place_of: torch.Tensor, wts: torch.Tensor, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = sum_k wts[t, k] * y[place_of[t, k]] (+ extra[t]) -> fp32 [T, W]."""
+def moe_combine(y, place_of: Optional[torch.Tensor] = None, wts: Optional[torch.Tensor] = None, extra: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = sum_k wts[t, k] * y[place_of[t, k]] (+ extra[t]) -> fp32 [T, W]; y may be a MoeSum holding all four."""
+    if isinstance(y, MoeSum):
+        y, place_of, wts, extra = y.y, y.place_of, y.wts, y.extra
     _dev(y, torch.float32, "moe_combine.y"); _dev(wts, torch.float32, "moe_combine.wts")
     T, top = wts.shape
     W = y.shape[1]

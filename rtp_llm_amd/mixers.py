@@ -365,8 +365,9 @@ class RoutedExperts:
         self.w_gate_up, self.w_down = torch.stack(gu).contiguous(), torch.stack(dn).contiguous()
         self.shared, self.act = shared, hops.ACTIVATIONS[act]
 
-    def forward(self, h: torch.Tensor, logits: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """logits: the router's fp32 logits [T, experts] when the caller has computed them (in a linear shared with other projections of h)."""
+    def forward(self, h: torch.Tensor, logits: Optional[torch.Tensor] = None, defer: bool = False):
+        """logits: the router's fp32 logits [T, experts] when the caller has computed them (in a linear shared with other projections of h).
+        defer: return the parts of the weighted sum (hybrid_ops.MoeSum) for a residual kernel that forms it, instead of the summed tensor."""
         r = self.router
         if logits is None:
             logits = hops.dense_linear(h, self.w_router, out_dtype=torch.float32)
@@ -374,7 +375,8 @@ class RoutedExperts:
         n = ids.numel()
         a = hops.dense_grouped(h, self.w_gate_up, offs=offs, gather=src, tiles=tiles, rows=n, gated=True, act=self.act)
         y = hops.dense_grouped(a, self.w_down, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32)
-        return hops.moe_combine(y, place, wts, self.shared.forward(h) if self.shared is not None else None)
+        parts = hops.MoeSum(y, place, wts, self.shared.forward(h) if self.shared is not None else None)
+        return parts if defer else hops.moe_combine(parts)
 
 
 class GatedMLP:

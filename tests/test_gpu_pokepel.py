@@ -99,6 +99,24 @@ def test_gated_branches_join_the_stream():
         xd = x.to(DEV)                                          # the mixer's branch alone
         hops.residual_norm(xd, a.to(DEV), None, 1.0, w1.to(DEV), None, 1e-6, gate=gate.to(DEV))
         close(xd, x.double() + torch.sigmoid(gate[:, :W].double()) * a.double(), 1e-5)
+        # the second branch as a mixture's weighted sum formed inside the kernel (with and without a shared expert's output), also under a row gather
+        y, wts = torch.randn(21, W, generator=g), torch.rand(7, 3, generator=g)
+        place = torch.randperm(21, generator=g).to(torch.int32).view(7, 3)
+        mix = (wts.double()[:, :, None] * y.double()[place.long()]).sum(1)
+        for extra in (b, None):
+            ms = hops.MoeSum(y.to(DEV), place.to(DEV), wts.to(DEV), None if extra is None else extra.to(DEV))
+            want = mix + (0 if extra is None else extra.double())
+            close(hops.moe_combine(ms), want, 1e-5)
+            xd = x.to(DEV)
+            h1, _ = hops.residual_norm(xd, a.to(DEV), ms, 1.0, w1.to(DEV), None, 1e-6, gate=gate.to(DEV))
+            xn = x.double() + torch.sigmoid(gate[:, :W].double()) * a.double() + torch.sigmoid(gate[:, W:2 * W].double()) * want
+            close(xd, xn, 1e-5)
+            close(h1, O.rms_unit(xn, 1e-6) * w1.double(), 1e-4)
+            xd = x.to(DEV)
+            rows = torch.tensor([6, 2], dtype=torch.int32, device=DEV)
+            h3, _ = hops.residual_norm(xd, a.to(DEV), ms, 1.0, w1.to(DEV), None, 1e-6, gate=gate.to(DEV), rows=rows)
+            close(h3, (O.rms_unit(xn, 1e-6) * w1.double())[[6, 2]], 1e-4)
+            close(xd, x.double(), 0.0)
 
 
 def test_polynorm_activation():
