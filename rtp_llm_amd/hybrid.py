@@ -149,6 +149,7 @@ class HybridModel:
         if self.embed.shape != (cfg.vocab, cfg.width) or self.head.shape != (cfg.vocab, cfg.width):
             raise ValueError(f"embed {tuple(self.embed.shape)} / head {tuple(self.head.shape)} against vocab {cfg.vocab} width {cfg.width}")
         self.layers = []
+        self.n_mix = {}                                  # layer -> (columns, padded columns) of the mixer's inputs inside the layer's shared linear
         for i, L in enumerate(cfg.layers):
             p = f"l{i}."
             if L.kind == "attention":
@@ -187,6 +188,14 @@ class HybridModel:
                     gate_w = torch.cat([gate_w, rw], 0).contiguous()
                     gate_b = torch.cat([gate_b, torch.zeros(rw.shape[0], dtype=dtype, device=self.device)], 0).contiguous()
             n2 = get(p + "norm2") if mlp is not None and not cfg.shared_norm else None
+            if gate_w is not None and cfg.shared_norm and isinstance(mixer, (LatentAttention, Retention)):
+                # every projection of the layer's one normed input in ONE linear: [mixer inputs (padded to 4 columns) | gates | router]
+                pad = (-mixer.w_in.shape[0]) % 4
+                zrow = torch.zeros(pad, cfg.width, dtype=dtype, device=self.device)
+                self.n_mix[i] = (mixer.w_in.shape[0], mixer.w_in.shape[0] + pad)
+                gate_b = torch.cat([torch.zeros(mixer.w_in.shape[0] + pad, dtype=dtype, device=self.device), gate_b], 0).contiguous()
+                gate_w = torch.cat([mixer.w_in, zrow, gate_w], 0).contiguous()
+                mixer.w_in = None                      # lives on as the leading rows of the shared weight
             self.layers.append((L, mixer, mlp, get(p + "norm1"), n2, gate_w, gate_b))
         self.has_state = any(L.kind not in ("attention", "latent_attention") for L in cfg.layers)
 
@@ -225,14 +234,25 @@ class HybridModel:
         cfg = self.cfg
         x = hops.embed(batch.tokens, self.embed)
         a = b = g = None
-        for (L, mixer, mlp, n1, n2, gate_w, gate_b), cache in zip(self.layers, caches):
+        shared = self.n_mix
+        for i, ((L, mixer, mlp, n1, n2, gate_w, gate_b), cache) in enumerate(zip(self.layers, caches)):
             h1, h2 = hops.residual_norm(x, a, b, cfg.residual_mult, n1, n2, cfg.eps, weight_offset=cfg.norm_offset, gate=g)
             if collect is not None and a is not None:
                 collect.append(x.clone())
             if cfg.shared_norm:
                 h2 = h1
-            g = hops.dense_linear(h1, gate_w, gate_b, out_dtype=torch.float32) if gate_w is not None else None
-            a = mixer.forward(h1, batch, *cache) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache)
+            if i in shared:                            # the mixer's projections are the leading rows of the gates' weight
+                n_in, n_pad = shared[i]
+                if h1.shape[0] <= 16:                  # decode-sized steps: one launch streams the whole weight
+                    g = hops.dense_linear(h1, gate_w, gate_b, out_dtype=torch.float32)
+                    proj, g = g[:, :n_in], g[:, n_pad:]
+                else:                                  # prompt portions: the tile kernel is faster on the two halves (measured: 0.6 ms of a 2048-token prefill)
+                    proj = hops.dense_linear(h1, gate_w[:n_in], out_dtype=torch.float32)
+                    g = hops.dense_linear(h1, gate_w[n_pad:], gate_b[n_pad:], out_dtype=torch.float32)
+                a = mixer.forward(h1, batch, *cache, proj=proj) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache, proj=proj)
+            else:
+                g = hops.dense_linear(h1, gate_w, gate_b, out_dtype=torch.float32) if gate_w is not None else None
+                a = mixer.forward(h1, batch, *cache) if isinstance(cache, tuple) else mixer.forward(h1, batch, cache)
             if mlp is None:
                 b = None
             elif g is not None and isinstance(mlp, RoutedExperts):

@@ -255,12 +255,14 @@ class LatentAttention:
                                                num_pages))
         return self._geom[1], self._geom[2]
 
-    def forward(self, h: torch.Tensor, batch: StepBatch, cache: torch.Tensor, _values=None) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch: StepBatch, cache: torch.Tensor, _values=None, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """proj: h w_in^T in fp32 when the caller has computed it (as columns of a linear shared with other projections of h)."""
         s = self.spec
         H, R = s.heads, s.kv_rank
         ageom, lgeom = self.geometry(batch.block_table.shape[1], cache.shape[0])
         T = h.shape[0]
-        proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        if proj is None:
+            proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
         qn = torch.empty(T, H * s.dim, dtype=self.act, device=h.device)
         qabs = torch.empty(T, H * self.padded, dtype=torch.float32, device=h.device)
         hops.latent_prep(proj, self.doff, lgeom, self.freq, self.mag, self.c_norm, self.eps, batch.pos, batch.seq, batch.block_table, qn, qabs, cache)
@@ -306,9 +308,11 @@ class Retention:
         s = self.spec
         return (s.heads, s.dim, s.vdim)
 
-    def forward(self, h: torch.Tensor, batch: StepBatch, state: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, batch: StepBatch, state: torch.Tensor, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """proj: h w_in^T in fp32 when the caller has computed it (as columns of a linear shared with other projections of h)."""
         s = self.spec
-        proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
+        if proj is None:
+            proj = hops.dense_linear(h, self.w_in, out_dtype=torch.float32)
         rot = s.rot
         hops.rotary(proj, [(self.qo, s.heads, s.dim, 1.0), (self.ko, s.heads, s.dim, 1.0 / math.sqrt(s.dim))], rot.dims if rot else 0,
                     hops.LAYOUTS[rot.layout] if rot else 0, self.freq, self.mag, batch.pos)
