@@ -389,7 +389,7 @@ def kernel_table_pokepel(s, dev, prompt):
         h = bf(T_, W)
         z = f32(T_, E) * 2
         gr = moe["router"]["groups"]
-        t = timed_k(lambda: hops.moe_align(hops.moe_route(z, gr["count"], gr["keep"], top)[0], E))
+        t = timed_k(lambda: hops.moe_route_sorted(z, E, gr["count"], gr["keep"], top))
         add("pokepel", "moe route + sort", f"T={T_} E={E} top={top}", t, T_ * (E * 4 + top * 16), 0, VALU_F32)
         ids, wts = hops.moe_route(z, gr["count"], gr["keep"], top)
         offs, src, place, tiles = hops.moe_align(ids, E)
@@ -402,8 +402,9 @@ def kernel_table_pokepel(s, dev, prompt):
         t = timed_k(lambda: hops.dense_grouped(a, wdn, offs=offs, tiles=tiles, rows=n, out_dtype=torch.float32))
         add("pokepel", "dense_grouped experts down", f"M={T_}x{top} E={E} ({used} used) N={W} K={fe}", t, used * fe * W * 2 + n * (fe * 2 + W * 4), 2.0 * n * fe * W, MFMA_BF16)
         y, extra = f32(n, W), f32(T_, W)
-        t = timed_k(lambda: hops.moe_combine(y, place, wts, extra))
-        add("pokepel", "moe weighted sum + shared", f"T={T_} top={top} W={W}", t, (n + 2 * T_) * W * 4, 0, VALU_F32)
+        xs_, as_, gt_, w1_ = f32(T_, W), f32(T_, W), f32(T_, 2 * W), bf(W)
+        t = timed_k(lambda: hops.residual_norm(xs_, as_, hops.MoeSum(y, place, wts, extra), 1.0, w1_, None, 1e-6, gate=gt_))
+        add("pokepel", "gated residual + mixture sum + norm", f"T={T_} top={top} W={W}", t, (n + 7 * T_) * W * 4 + T_ * W * 2, 0, VALU_F32)
         ffa = fe * top
         wd_gu = hops.group_gate_up(bf(ffa, W), bf(ffa, W))
         t = timed_k(lambda: hops.dense_linear(h, wd_gu, gated=True, act=hops.ACT_RELU))
